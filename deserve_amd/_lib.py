@@ -1,0 +1,124 @@
+"""ctypes binding of libdskv.so, the C ABI declared in include/dskv.h.
+
+The library is the only compute path: if it is missing, loading raises and
+every operator of this package fails loudly - there is no fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_void_p
+from typing import Optional
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdskv.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+F32, F16, BF16 = 0, 1, 2
+
+_lib: Optional[ctypes.CDLL] = None
+
+# name -> (restype, argtypes); mirrors include/dskv.h one to one
+_SIGNATURES = {
+    "dskv_last_error": (c_char_p, []),
+    "dskv_version": (c_int32, []),
+    "dskv_append_paged_kv": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                       c_int32, c_void_p]),
+    "dskv_gather_pages": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int64,
+                                    c_int64, c_int64, c_int64, c_void_p]),
+    "dskv_scatter_pages": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int64,
+                                     c_int64, c_int64, c_int64, c_void_p]),
+    "dskv_decode_plan_bound": (c_int64, [c_int32, c_int64]),
+    "dskv_decode_plan": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                   c_int32, c_void_p, c_int64, POINTER(c_int32), POINTER(c_int64),
+                                   POINTER(c_int64)]),
+    "dskv_decode_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_int32, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
+                                   c_int32, c_float, c_int32, c_void_p]),
+    "dskv_prefill_plan_bound": (c_int64, [c_int32, c_int64]),
+    "dskv_prefill_plan": (c_int32, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_int64,
+                                    POINTER(c_int32)]),
+    "dskv_prefill_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                    c_int32, c_int32, c_float, c_int32, c_int32, c_void_p]),
+    "dskv_apply_rope": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
+                                  c_void_p]),
+    "dskv_swap_slice": (c_int32, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p,
+                                  c_void_p, c_void_p]),
+    "dskv_swap_create": (c_int32, [POINTER(c_void_p), c_int64]),
+    "dskv_swap_destroy": (c_int32, [c_void_p]),
+    "dskv_swap_out_async": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                      c_int64, c_int64, c_void_p]),
+    "dskv_swap_in_async": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                     c_int64, c_int64, c_void_p]),
+    "dskv_swap_exchange_async": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_int32, c_int32, c_int64, c_int64, c_void_p]),
+    "dskv_swap_wait": (c_int32, [c_void_p]),
+    "dskv_swap_fence": (c_int32, [c_void_p, c_void_p]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def build(force: bool = True) -> str:
+    """Compile csrc/ for gfx950 into libdskv.so (hipcc cross-compiles without a GPU)."""
+    cmd = ["make", "-C", CSRC_DIR, "-j8", f"OUT={LIB_PATH}"]
+    if force:
+        cmd.insert(1, "-B")
+    subprocess.check_call(cmd)
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension is not built "
+                "(run `python -c 'import __graft_entry__ as g; g.build()'`); "
+                "deserve_amd has no other compute path")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    msg = lib().dskv_last_error()
+    return msg.decode() if msg else ""
+
+
+def check(rc: int, what: str = "dskv") -> None:
+    """0 ok; negative = argument error -> ValueError; positive = HIP error -> RuntimeError."""
+    if rc == 0:
+        return
+    msg = f"{what}: {last_error()} (code {rc})"
+    if rc < 0:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def dtype_code(dtype) -> int:
+    import torch
+
+    try:
+        return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported KV dtype {dtype}") from None
+
+
+def ptr(t) -> int:
+    """Raw address of a tensor's first element (0 for None)."""
+    return 0 if t is None else t.data_ptr()
+
+
+def current_stream() -> int:
+    import torch
+
+    return torch.cuda.current_stream().cuda_stream

@@ -1,0 +1,129 @@
+// 16-token K/V tile movement shared by the decode and prefill attention kernels
+// (head_dim 128, 16-bit elements, one wavefront per kv head).
+//
+// Lane roles, with g = lane / 16 and c = lane % 16:
+//   K: lane holds dims kk*32 + g*8 .. +8 (kk = 0..3) of tile row c, which is
+//      token row_to_token(c) of the tile - the A operand of the 16x16x32 MFMA.
+//   V: lane holds the 16-byte chunk c of tile tokens g, g+4, g+8, g+12; the tile
+//      is written to LDS as loaded and read back column-wise as the A operand of
+//      the 16x16x16 MFMA (4 tokens g, g+4, g+8, g+12 of one dim per lane).
+// The token permutation makes the four lane groups read neighbouring LDS rows of
+// a 288-byte-pitch tile, which is bank-conflict free.
+#pragma once
+
+#include "mfma.h"
+
+namespace dskv {
+
+constexpr int kTile = 16;                 // tokens per MFMA tile
+constexpr int kHeadDim = 128;             // the MFMA kernels are specialised for D = 128
+constexpr int kVPitch = 288;              // bytes per V row in LDS (256 + 32 pad)
+constexpr int kVTileBytes = kTile * kVPitch;
+constexpr int kBufferFlags = 0x00020000;  // raw buffer descriptor word 3 for 32-bit data
+constexpr int kOutOfRange = 0x7FFF0000;   // byte offset no page reaches: reads as zero, moves nothing
+
+// MFMA row m of a tile holds token (m >> 2) + 4 * (m & 3) of that tile.
+__device__ __forceinline__ int row_to_token(int m) { return (m >> 2) + ((m & 3) << 2); }
+
+struct TileRegs {
+    u32x4 k[4];
+    u32x4 v[4];
+};
+
+// One request's paged K/V of one layer as seen by one wave (one kv head).
+struct KvView {
+    const char *pages;           // layer base: (num_pages, 2, P, Hkv, 128) 16-bit
+    const int32_t *page_ids;     // this request's block-table entries
+    int page_shift;              // log2(page_size)
+    int row_bytes;               // one token, all kv heads
+    int half_bytes;              // K half of a page
+    long page_bytes;
+    int head_off;                // byte offset of this wave's kv head inside a token row
+};
+
+// Loads tile [t, t + 16) of a request whose valid tokens end at t_end.  Issued
+// unconditionally (so the count of loads in flight is static); nothing past
+// t_end is fetched.
+template <bool kPageCoversTile>
+__device__ __forceinline__ void load_kv_tile(const KvView &kv, int t, int t_end, int g, int c,
+                                             TileRegs &r)
+{
+    const int k_tok = row_to_token(c);
+    if (kPageCoversTile) {
+        // One page holds the whole tile: address it through a buffer descriptor
+        // of that page.  Rows at or past t_end get an offset outside the page
+        // and a tile past the end gets an empty descriptor: such lanes read zero
+        // and generate no memory traffic.
+        const int page_size = 1 << kv.page_shift;
+        const int last_page = max((t_end - 1) >> kv.page_shift, 0);
+        const long page = kv.page_ids[min(t >> kv.page_shift, last_page)];
+        const int slot_off = (t & (page_size - 1)) * kv.row_bytes;
+        __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(kv.pages) + page * kv.page_bytes, 0,
+            t < t_end ? (int)kv.page_bytes : 0, kBufferFlags);
+        const int ko = (t + k_tok < t_end) ? slot_off + k_tok * kv.row_bytes + kv.head_off + g * 16
+                                           : kOutOfRange;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+            r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int vo = (t + g + 4 * i < t_end)
+                               ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes +
+                                     kv.head_off + c * 16
+                               : kOutOfRange;
+            r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, 0);
+        }
+    } else {
+        // Pages smaller than a tile: every lane resolves its own page.  Tokens
+        // past the end are clamped to the last valid one; the consumer masks
+        // their scores and zeroes their V rows.
+        const int page_mask = (1 << kv.page_shift) - 1;
+        const int t_last = max(t_end - 1, 0);
+        const int tk = min(t + k_tok, t_last);
+        const long kpage = kv.page_ids[tk >> kv.page_shift];
+        const char *kp = kv.pages + kpage * kv.page_bytes + (long)(tk & page_mask) * kv.row_bytes +
+                         kv.head_off + g * 16;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) r.k[kk] = *reinterpret_cast<const u32x4 *>(kp + kk * 64);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int tv = min(t + g + 4 * i, t_last);
+            const long vpage = kv.page_ids[tv >> kv.page_shift];
+            const char *vp = kv.pages + vpage * kv.page_bytes + kv.half_bytes +
+                             (long)(tv & page_mask) * kv.row_bytes + kv.head_off + c * 16;
+            r.v[i] = *reinterpret_cast<const u32x4 *>(vp);
+        }
+    }
+}
+
+// V tile -> this wave's LDS tile.  Rows at or past t_end must be zero (their
+// probabilities are zero, but 0 * garbage is not): the buffer-descriptor path
+// already delivers zeros, the clamped path zeroes them here.  The tile is
+// private to the wave; LDS executes a wave's accesses in order, the barriers
+// only pin the compiler's order.
+template <bool kPageCoversTile>
+__device__ __forceinline__ void stage_v_tile(char *lds, const TileRegs &r, int t, int t_end, int g,
+                                             int c)
+{
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        u32x4 vv = r.v[i];
+        if (!kPageCoversTile && t + g + 4 * i >= t_end) vv = u32x4{0, 0, 0, 0};
+        *reinterpret_cast<u32x4 *>(lds + (g + 4 * i) * kVPitch + c * 16) = vv;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// A operand of the P.V MFMA for dim tile dt: V[token g + 4j][dim dt*16 + c], j = 0..3.
+__device__ __forceinline__ u32x2 read_v_operand(const char *lds, int dt, int g, int c)
+{
+    const uint16_t *vc = reinterpret_cast<const uint16_t *>(lds + g * kVPitch) + dt * 16 + c;
+    const uint32_t a0 = vc[0] | ((uint32_t)vc[4 * (kVPitch / 2)] << 16);
+    const uint32_t a1 = vc[8 * (kVPitch / 2)] | ((uint32_t)vc[12 * (kVPitch / 2)] << 16);
+    return u32x2{a0, a1};
+}
+
+}  // namespace dskv

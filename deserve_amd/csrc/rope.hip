@@ -1,0 +1,156 @@
+// Rotary position embedding on the ragged q/k of one step, adjacent-pair
+// ("interleaved") convention: (x[2j], x[2j+1]) is rotated by
+// pos * theta^(-2j/D) with pos = offsets[request] + index within the request.
+// Elementwise, HBM-bound; one workgroup per token.  A thread owns one 16-byte
+// chunk column of the head dimension, evaluates its sin/cos once and walks the
+// heads, so the transcendental work is per (token, dim pair), not per head.
+#include "common.h"
+
+#include <math.h>
+
+namespace dskv {
+
+template <int DT> struct Chunk;   // 16 bytes <-> fp32 lanes
+template <> struct Chunk<DSKV_F32> {
+    static constexpr int kElems = 4;
+    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = __builtin_bit_cast(float, raw[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = __builtin_bit_cast(uint32_t, f[i]);
+        return r;
+    }
+};
+template <> struct Chunk<DSKV_F16> {
+    static constexpr int kElems = 8;
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            h2 p = __builtin_bit_cast(h2, raw[i]);
+            f[2 * i] = (float)p[0];
+            f[2 * i + 1] = (float)p[1];
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            h2 p = {(_Float16)f[2 * i], (_Float16)f[2 * i + 1]};
+            r[i] = __builtin_bit_cast(uint32_t, p);
+        }
+        return r;
+    }
+};
+template <> struct Chunk<DSKV_BF16> {
+    static constexpr int kElems = 8;
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[2 * i] = __builtin_bit_cast(float, raw[i] << 16);
+            f[2 * i + 1] = __builtin_bit_cast(float, raw[i] & 0xFFFF0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float *f) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            b2 p = {(__bf16)f[2 * i], (__bf16)f[2 * i + 1]};
+            r[i] = __builtin_bit_cast(uint32_t, p);
+        }
+        return r;
+    }
+};
+
+template <int DT>
+__global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, char *__restrict__ k_out,
+                                                   const char *__restrict__ q,
+                                                   const char *__restrict__ k,
+                                                   const int32_t *__restrict__ qo_indptr,
+                                                   const int32_t *__restrict__ offsets, int batch,
+                                                   int n_qo_heads, int n_kv_heads, int head_dim,
+                                                   float theta)
+{
+    typedef Chunk<DT> C;
+    constexpr int E = C::kElems;
+    const int t = blockIdx.x;
+    int lo = 0, hi = batch;   // largest b with qo_indptr[b] <= t
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (qo_indptr[mid] <= t) lo = mid; else hi = mid;
+    }
+    if (t >= qo_indptr[lo + 1]) return;   // token not covered by the metadata
+    const float pos = (float)(offsets[lo] + (t - qo_indptr[lo]));
+
+    const int cols = head_dim / E;           // 16-byte chunks per head row
+    const int col = threadIdx.x % cols;
+    const int head_lane = threadIdx.x / cols;
+    const int head_lanes = 256 / cols;
+    if (head_lane >= head_lanes) return;
+
+    float cs[E / 2], sn[E / 2];
+#pragma unroll
+    for (int j = 0; j < E / 2; j++) {
+        const int pair = col * (E / 2) + j;
+        // theta^(-2*pair/D), evaluated as the reference's table does: 1 / theta^(2*pair/D)
+        const float inv_freq = 1.0f / powf(theta, (float)(2 * pair) / (float)head_dim);
+        sincosf(pos * inv_freq, &sn[j], &cs[j]);
+    }
+    const long row_bytes = (long)head_dim * (16 / E);
+    const int total_heads = n_qo_heads + n_kv_heads;
+    for (int h = head_lane; h < total_heads; h += head_lanes) {
+        const bool is_q = h < n_qo_heads;
+        const long off = is_q ? ((long)t * n_qo_heads + h) * row_bytes
+                              : ((long)t * n_kv_heads + (h - n_qo_heads)) * row_bytes;
+        const char *src = (is_q ? q : k) + off + col * 16;
+        char *dst = (is_q ? q_out : k_out) + off + col * 16;
+        float f[E];
+        C::unpack(*reinterpret_cast<const u32x4 *>(src), f);
+#pragma unroll
+        for (int j = 0; j < E / 2; j++) {
+            const float re = f[2 * j], im = f[2 * j + 1];
+            f[2 * j] = re * cs[j] - im * sn[j];
+            f[2 * j + 1] = re * sn[j] + im * cs[j];
+        }
+        *reinterpret_cast<u32x4 *>(dst) = C::pack(f);
+    }
+}
+
+}  // namespace dskv
+
+extern "C" int dskv_apply_rope(void *q_out, void *k_out, const void *q, const void *k,
+                               const int32_t *qo_indptr, const int32_t *offsets, int32_t batch,
+                               int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
+                               int32_t head_dim, float rope_theta, int32_t dtype, void *stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(batch >= 0 && nnz >= 0, "apply_rope: negative batch/nnz");
+    if (batch == 0 || nnz == 0) return 0;
+    DSKV_REQUIRE(q_out && k_out && q && k && qo_indptr && offsets, "apply_rope: null pointer argument");
+    DSKV_REQUIRE(dtype == DSKV_F32 || dtype == DSKV_F16 || dtype == DSKV_BF16,
+                 "apply_rope: unknown dtype %d", dtype);
+    const int elems = dtype == DSKV_F32 ? 4 : 8;
+    DSKV_REQUIRE(head_dim > 0 && head_dim % elems == 0 && head_dim / elems <= 256,
+                 "apply_rope: head_dim %d must be a multiple of %d and at most %d", head_dim, elems,
+                 256 * elems);
+    DSKV_REQUIRE(n_qo_heads > 0 && n_kv_heads > 0, "apply_rope: bad head counts");
+    DSKV_REQUIRE(rope_theta > 0.f, "apply_rope: rope_theta must be positive");
+    DSKV_REQUIRE(((uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)q | (uintptr_t)k) % 16 == 0,
+                 "apply_rope: q/k must be 16-byte aligned");
+    
+    hipStream_t s = (hipStream_t)stream;
+#define DSKV_LAUNCH_ROPE(DT)                                                                    \
+    hipLaunchKernelGGL((rope_kernel<DT>), dim3((unsigned)nnz), dim3(256), 0, s, (char *)q_out,  \
+                       (char *)k_out, (const char *)q, (const char *)k, qo_indptr, offsets,     \
+                       batch, n_qo_heads, n_kv_heads, head_dim, rope_theta)
+    if (dtype == DSKV_F32) DSKV_LAUNCH_ROPE(DSKV_F32);
+    else if (dtype == DSKV_F16) DSKV_LAUNCH_ROPE(DSKV_F16);
+    else DSKV_LAUNCH_ROPE(DSKV_BF16);
+#undef DSKV_LAUNCH_ROPE
+    DSKV_LAUNCH_CHECK("rope_kernel");
+    return 0;
+}

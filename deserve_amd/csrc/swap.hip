@@ -1,0 +1,326 @@
+// KV swap between the HBM page pool and pinned host DRAM.
+//
+// Bound: the host link (PCIe); HBM-side staging traffic is overhead.
+//
+// Two forms:
+//  * dskv_swap_slice - a contiguous slice of pool pages of every layer; each
+//    layer's slice is one contiguous run, so it is one async copy per layer and
+//    direction, split over two caller streams.
+//  * the scattered-page engine - pages named by a block table are packed by a
+//    gather kernel into a contiguous staging buffer and leave in one large
+//    async copy per staging chunk (and the reverse for swap-in).  Two staging
+//    buffers and two streams per direction keep a gather and a copy in flight
+//    at once; the two directions have their own streams so D2H and H2D traffic
+//    of an exchange use both halves of the full-duplex link.
+#include "common.h"
+
+#include <algorithm>
+#include <new>
+#include <vector>
+
+struct dskv_swap {
+    int device = 0;
+    int64_t staging_bytes = 0;
+    // [direction: 0 = out (D2H), 1 = in (H2D)][ping-pong]
+    hipStream_t stream[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+    void *staging[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+    hipEvent_t dir_done[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+    bool dir_used[2] = {false, false};
+    hipEvent_t ready = nullptr;        // caller's stream reached the call
+    hipEvent_t ids_ready = nullptr;    // page ids have landed on the device
+    hipEvent_t gathered[2] = {nullptr, nullptr};   // exchange: chunk left the pool
+    hipEvent_t fence = nullptr;
+    // page-id arena: pinned host mirror + device copy, bump-allocated, reset on wait
+    int32_t *ids_host = nullptr;
+    int32_t *ids_dev = nullptr;
+    int64_t ids_capacity = 0;
+    int64_t ids_used = 0;
+};
+
+namespace dskv {
+
+constexpr int64_t kIdsCapacity = int64_t(1) << 20;
+
+static int check_geometry(const char *who, int32_t n_pages, int32_t n_layers,
+                          int64_t layer_stride_bytes, int64_t page_bytes)
+{
+    DSKV_REQUIRE(n_pages >= 0 && n_layers >= 0, "%s: negative sizes", who);
+    DSKV_REQUIRE(page_bytes > 0 && page_bytes % 16 == 0,
+                 "%s: page_bytes (%lld) must be a positive multiple of 16", who,
+                 (long long)page_bytes);
+    DSKV_REQUIRE(layer_stride_bytes >= page_bytes && layer_stride_bytes % 16 == 0,
+                 "%s: bad layer stride %lld", who, (long long)layer_stride_bytes);
+    return 0;
+}
+
+static int wait_all(dskv_swap *h)
+{
+    for (int d = 0; d < 2; d++)
+        for (int i = 0; i < 2; i++) DSKV_HIP(hipStreamSynchronize(h->stream[d][i]));
+    h->ids_used = 0;
+    return 0;
+}
+
+// Copy the caller's page ids into the arena and start their upload on `s`.
+static int stage_ids(dskv_swap *h, const int32_t *ids, int32_t n, hipStream_t s, int32_t **dev_out)
+{
+    DSKV_REQUIRE(n <= h->ids_capacity, "swap: %d page ids exceed the engine's limit of %lld", n,
+                 (long long)h->ids_capacity);
+    if (h->ids_used + n > h->ids_capacity) {
+        int rc = wait_all(h);   // arena full: drain, then start over
+        if (rc) return rc;
+    }
+    int32_t *host = h->ids_host + h->ids_used;
+    int32_t *dev = h->ids_dev + h->ids_used;
+    std::copy(ids, ids + n, host);
+    h->ids_used += n;
+    DSKV_HIP(hipMemcpyAsync(dev, host, (size_t)n * sizeof(int32_t), hipMemcpyHostToDevice, s));
+    *dev_out = dev;
+    return 0;
+}
+
+// Both streams of direction `dir` wait for: the caller's stream, the id upload,
+// and everything previously enqueued in the opposite direction (an earlier
+// swap-out may still be reading pages that this swap-in is about to overwrite,
+// and the other way round).
+static int open_direction(dskv_swap *h, int dir, hipStream_t after, hipStream_t ids_stream)
+{
+    DSKV_HIP(hipEventRecord(h->ready, after));
+    DSKV_HIP(hipEventRecord(h->ids_ready, ids_stream));
+    for (int i = 0; i < 2; i++) {
+        hipStream_t s = h->stream[dir][i];
+        DSKV_HIP(hipStreamWaitEvent(s, h->ready, 0));
+        if (s != ids_stream) DSKV_HIP(hipStreamWaitEvent(s, h->ids_ready, 0));
+        if (h->dir_used[1 - dir])
+            for (int j = 0; j < 2; j++)
+                DSKV_HIP(hipStreamWaitEvent(s, h->dir_done[1 - dir][j], 0));
+    }
+    return 0;
+}
+
+static int close_direction(dskv_swap *h, int dir)
+{
+    for (int i = 0; i < 2; i++) DSKV_HIP(hipEventRecord(h->dir_done[dir][i], h->stream[dir][i]));
+    h->dir_used[dir] = true;
+    return 0;
+}
+
+}  // namespace dskv
+
+extern "C" int dskv_swap_slice(void *slice_base, int64_t layer_stride_bytes, int64_t slice_bytes,
+                               int32_t n_layers, void *host_to, const void *host_from,
+                               void *stream0, void *stream1)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(n_layers >= 0 && slice_bytes >= 0, "swap_slice: negative sizes");
+    if (n_layers == 0 || slice_bytes == 0 || (!host_to && !host_from)) return 0;
+    DSKV_REQUIRE(slice_base, "swap_slice: null slice pointer");
+    DSKV_REQUIRE(layer_stride_bytes >= slice_bytes, "swap_slice: layer stride %lld < slice bytes %lld",
+                 (long long)layer_stride_bytes, (long long)slice_bytes);
+    const int mid = n_layers / 2;
+    for (int l = 0; l < n_layers; l++) {
+        hipStream_t s = (hipStream_t)(l < mid ? stream0 : stream1);
+        char *dev = (char *)slice_base + (int64_t)l * layer_stride_bytes;
+        if (host_to)
+            DSKV_HIP(hipMemcpyAsync((char *)host_to + (int64_t)l * slice_bytes, dev,
+                                    (size_t)slice_bytes, hipMemcpyDeviceToHost, s));
+        if (host_from)
+            DSKV_HIP(hipMemcpyAsync(dev, (const char *)host_from + (int64_t)l * slice_bytes,
+                                    (size_t)slice_bytes, hipMemcpyHostToDevice, s));
+    }
+    return 0;
+}
+
+extern "C" int dskv_swap_create(dskv_swap_t **handle, int64_t staging_bytes)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(handle, "swap_create: null handle pointer");
+    DSKV_REQUIRE(staging_bytes >= (1 << 20) && staging_bytes % 16 == 0,
+                 "swap_create: staging_bytes (%lld) must be >= 1 MiB and a multiple of 16",
+                 (long long)staging_bytes);
+    dskv_swap *h = new (std::nothrow) dskv_swap();
+    DSKV_REQUIRE(h, "swap_create: out of host memory");
+    *handle = nullptr;
+#define DSKV_CREATE(expr)                                                   \
+    do {                                                                    \
+        hipError_t e_ = (expr);                                             \
+        if (e_ != hipSuccess) {                                             \
+            set_error("%s failed: %s", #expr, hipGetErrorString(e_));       \
+            dskv_swap_destroy(h);                                           \
+            return (int)e_;                                                 \
+        }                                                                   \
+    } while (0)
+    DSKV_CREATE(hipGetDevice(&h->device));
+    h->staging_bytes = staging_bytes;
+    for (int d = 0; d < 2; d++)
+        for (int i = 0; i < 2; i++) {
+            DSKV_CREATE(hipStreamCreateWithFlags(&h->stream[d][i], hipStreamNonBlocking));
+            DSKV_CREATE(hipMalloc(&h->staging[d][i], (size_t)staging_bytes));
+            DSKV_CREATE(hipEventCreateWithFlags(&h->dir_done[d][i], hipEventDisableTiming));
+        }
+    DSKV_CREATE(hipEventCreateWithFlags(&h->ready, hipEventDisableTiming));
+    DSKV_CREATE(hipEventCreateWithFlags(&h->ids_ready, hipEventDisableTiming));
+    DSKV_CREATE(hipEventCreateWithFlags(&h->fence, hipEventDisableTiming));
+    for (int i = 0; i < 2; i++)
+        DSKV_CREATE(hipEventCreateWithFlags(&h->gathered[i], hipEventDisableTiming));
+    h->ids_capacity = kIdsCapacity;
+    DSKV_CREATE(hipHostMalloc((void **)&h->ids_host, (size_t)h->ids_capacity * sizeof(int32_t),
+                              hipHostMallocDefault));
+    DSKV_CREATE(hipMalloc((void **)&h->ids_dev, (size_t)h->ids_capacity * sizeof(int32_t)));
+#undef DSKV_CREATE
+    *handle = h;
+    return 0;
+}
+
+extern "C" int dskv_swap_destroy(dskv_swap_t *h)
+{
+    if (!h) return 0;
+    for (int d = 0; d < 2; d++)
+        for (int i = 0; i < 2; i++) {
+            if (h->stream[d][i]) {
+                (void)hipStreamSynchronize(h->stream[d][i]);
+                (void)hipStreamDestroy(h->stream[d][i]);
+            }
+            if (h->staging[d][i]) (void)hipFree(h->staging[d][i]);
+            if (h->dir_done[d][i]) (void)hipEventDestroy(h->dir_done[d][i]);
+        }
+    if (h->ready) (void)hipEventDestroy(h->ready);
+    if (h->ids_ready) (void)hipEventDestroy(h->ids_ready);
+    if (h->fence) (void)hipEventDestroy(h->fence);
+    for (int i = 0; i < 2; i++)
+        if (h->gathered[i]) (void)hipEventDestroy(h->gathered[i]);
+    if (h->ids_host) (void)hipHostFree(h->ids_host);
+    if (h->ids_dev) (void)hipFree(h->ids_dev);
+    delete h;
+    return 0;
+}
+
+extern "C" int dskv_swap_out_async(dskv_swap_t *h, void *host_dst, const void *pool,
+                                   const int32_t *page_ids_host, int32_t n_pages, int32_t n_layers,
+                                   int64_t layer_stride_bytes, int64_t page_bytes,
+                                   void *after_stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_out: null handle");
+    int rc = check_geometry("swap_out", n_pages, n_layers, layer_stride_bytes, page_bytes);
+    if (rc) return rc;
+    const int64_t rows = (int64_t)n_pages * n_layers;
+    if (rows == 0) return 0;
+    DSKV_REQUIRE(host_dst && pool && page_ids_host, "swap_out: null pointer argument");
+    const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
+    DSKV_REQUIRE(rows_per_chunk >= 1, "swap_out: a page (%lld bytes) does not fit the staging buffer",
+                 (long long)page_bytes);
+    int32_t *ids_dev = nullptr;
+    if ((rc = stage_ids(h, page_ids_host, n_pages, h->stream[0][0], &ids_dev))) return rc;
+    if ((rc = open_direction(h, 0, (hipStream_t)after_stream, h->stream[0][0]))) return rc;
+    int c = 0;
+    for (int64_t r0 = 0; r0 < rows; r0 += rows_per_chunk, c ^= 1) {
+        const int64_t r1 = std::min(rows, r0 + rows_per_chunk);
+        hipStream_t s = h->stream[0][c];
+        if ((rc = dskv_gather_pages(h->staging[0][c], pool, ids_dev, n_pages, n_layers,
+                                    layer_stride_bytes, page_bytes, r0, r1, s)))
+            return rc;
+        DSKV_HIP(hipMemcpyAsync((char *)host_dst + r0 * page_bytes, h->staging[0][c],
+                                (size_t)((r1 - r0) * page_bytes), hipMemcpyDeviceToHost, s));
+    }
+    return close_direction(h, 0);
+}
+
+extern "C" int dskv_swap_in_async(dskv_swap_t *h, void *pool, const void *host_src,
+                                  const int32_t *page_ids_host, int32_t n_pages, int32_t n_layers,
+                                  int64_t layer_stride_bytes, int64_t page_bytes,
+                                  void *after_stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_in: null handle");
+    int rc = check_geometry("swap_in", n_pages, n_layers, layer_stride_bytes, page_bytes);
+    if (rc) return rc;
+    const int64_t rows = (int64_t)n_pages * n_layers;
+    if (rows == 0) return 0;
+    DSKV_REQUIRE(host_src && pool && page_ids_host, "swap_in: null pointer argument");
+    const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
+    DSKV_REQUIRE(rows_per_chunk >= 1, "swap_in: a page (%lld bytes) does not fit the staging buffer",
+                 (long long)page_bytes);
+    int32_t *ids_dev = nullptr;
+    if ((rc = stage_ids(h, page_ids_host, n_pages, h->stream[1][0], &ids_dev))) return rc;
+    if ((rc = open_direction(h, 1, (hipStream_t)after_stream, h->stream[1][0]))) return rc;
+    int c = 0;
+    for (int64_t r0 = 0; r0 < rows; r0 += rows_per_chunk, c ^= 1) {
+        const int64_t r1 = std::min(rows, r0 + rows_per_chunk);
+        hipStream_t s = h->stream[1][c];
+        DSKV_HIP(hipMemcpyAsync(h->staging[1][c], (const char *)host_src + r0 * page_bytes,
+                                (size_t)((r1 - r0) * page_bytes), hipMemcpyHostToDevice, s));
+        if ((rc = dskv_scatter_pages(pool, h->staging[1][c], ids_dev, n_pages, n_layers,
+                                     layer_stride_bytes, page_bytes, r0, r1, s)))
+            return rc;
+    }
+    return close_direction(h, 1);
+}
+
+extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const void *host_src,
+                                        void *pool, const int32_t *page_ids_host, int32_t n_pages,
+                                        int32_t n_layers, int64_t layer_stride_bytes,
+                                        int64_t page_bytes, void *after_stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_exchange: null handle");
+    int rc = check_geometry("swap_exchange", n_pages, n_layers, layer_stride_bytes, page_bytes);
+    if (rc) return rc;
+    const int64_t rows = (int64_t)n_pages * n_layers;
+    if (rows == 0) return 0;
+    DSKV_REQUIRE(host_dst && host_src && pool && page_ids_host,
+                 "swap_exchange: null pointer argument");
+    const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
+    DSKV_REQUIRE(rows_per_chunk >= 1,
+                 "swap_exchange: a page (%lld bytes) does not fit the staging buffer",
+                 (long long)page_bytes);
+    int32_t *ids_dev = nullptr;
+    if ((rc = stage_ids(h, page_ids_host, n_pages, h->stream[0][0], &ids_dev))) return rc;
+    if ((rc = open_direction(h, 0, (hipStream_t)after_stream, h->stream[0][0]))) return rc;
+    if ((rc = open_direction(h, 1, (hipStream_t)after_stream, h->stream[0][0]))) return rc;
+    // host_dst == host_src is a round trip through one buffer (two microbatch
+    // rounds share their pinned buffer): dump-then-refill leaves the pages as
+    // they were, so only the dump is performed.
+    const bool same_buffer = host_dst == host_src;
+    int c = 0;
+    for (int64_t r0 = 0; r0 < rows; r0 += rows_per_chunk, c ^= 1) {
+        const int64_t r1 = std::min(rows, r0 + rows_per_chunk);
+        const size_t bytes = (size_t)((r1 - r0) * page_bytes);
+        hipStream_t so = h->stream[0][c], si = h->stream[1][c];
+        // the gather of chunk c-2 used gathered[c]; its scatter (stream si) already waited on it
+        if ((rc = dskv_gather_pages(h->staging[0][c], pool, ids_dev, n_pages, n_layers,
+                                    layer_stride_bytes, page_bytes, r0, r1, so)))
+            return rc;
+        DSKV_HIP(hipEventRecord(h->gathered[c], so));
+        DSKV_HIP(hipMemcpyAsync((char *)host_dst + r0 * page_bytes, h->staging[0][c], bytes,
+                                hipMemcpyDeviceToHost, so));
+        if (same_buffer) continue;
+        DSKV_HIP(hipMemcpyAsync(h->staging[1][c], (const char *)host_src + r0 * page_bytes, bytes,
+                                hipMemcpyHostToDevice, si));
+        DSKV_HIP(hipStreamWaitEvent(si, h->gathered[c], 0));   // pages of this chunk have left
+        if ((rc = dskv_scatter_pages(pool, h->staging[1][c], ids_dev, n_pages, n_layers,
+                                     layer_stride_bytes, page_bytes, r0, r1, si)))
+            return rc;
+    }
+    if ((rc = close_direction(h, 0))) return rc;
+    return close_direction(h, 1);
+}
+
+extern "C" int dskv_swap_wait(dskv_swap_t *h)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_wait: null handle");
+    return wait_all(h);
+}
+
+extern "C" int dskv_swap_fence(dskv_swap_t *h, void *stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_fence: null handle");
+    for (int d = 0; d < 2; d++)
+        for (int i = 0; i < 2; i++) {
+            DSKV_HIP(hipEventRecord(h->fence, h->stream[d][i]));
+            DSKV_HIP(hipStreamWaitEvent((hipStream_t)stream, h->fence, 0));
+        }
+    return 0;
+}

@@ -1,0 +1,117 @@
+"""Per-step CSR metadata for the paged kernels
+(deserve_worker/model/context/flash.py:17-120).
+
+For every request: current_len = start_pos + seqlen tokens are visible, the
+cache is extended to max(current_len, initial_seqlen) (a chunked prefill
+reserves the whole prompt up front), ceil(current_len / P) block-table entries
+are exposed and the last page holds (current_len - 1) % P + 1 tokens.
+
+The reference builds six small device tensors with a cat of B device slices and
+five host-to-device constructions per step.  Here all six arrays are laid out in
+ONE pinned host buffer and reach the device in ONE async copy; the device
+tensors of the context are views of that upload, and the host copies are kept
+(``host`` dict) so the attention planner never reads back from the device.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Sequence
+
+import numpy as np
+import torch
+
+from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+from deserve_amd.model.context.forward import PagedForwardCtx
+from deserve_amd.paged_ops import (BatchDecodeWithPagedKVCacheWrapper,
+                                   BatchPrefillWithPagedKVCacheWrapper)
+from deserve_amd.task import TaskData
+
+_FIELDS = ("indptr", "kv_page_indptr", "kv_last_page_lens", "offsets", "seqlens",
+           "kv_page_indices")
+
+
+def build_host_metadata(task_datas: Sequence[TaskData],
+                        kvcaches: Sequence[PagedKVCache]) -> Dict[str, np.ndarray]:
+    """The six int32 arrays on the host; extends the caches as a side effect."""
+    B = len(task_datas)
+    indptr = np.zeros(B + 1, np.int32)
+    kv_indptr = np.zeros(B + 1, np.int32)
+    last = np.zeros(B, np.int32)
+    offsets = np.zeros(B, np.int32)
+    seqlens = np.zeros(B, np.int32)
+    rows: List[np.ndarray] = []
+    for i, (task, cache) in enumerate(zip(task_datas, kvcaches)):
+        page_size = cache.pool.page_size
+        current_len = task.start_pos + task.seqlen
+        cache.extend(max(current_len, task.initial_seqlen))
+        exposed = -(-current_len // page_size)
+        rows.append(cache.page_table.retrieve()[:exposed].numpy())
+        last[i] = (current_len - 1) % page_size + 1
+        offsets[i] = task.start_pos
+        seqlens[i] = task.seqlen
+        indptr[i + 1] = indptr[i] + task.seqlen
+        kv_indptr[i + 1] = kv_indptr[i] + exposed
+    indices = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
+    return dict(indptr=indptr, kv_page_indptr=kv_indptr, kv_last_page_lens=last, offsets=offsets,
+                seqlens=seqlens, kv_page_indices=indices)
+
+
+def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device):
+    """One pinned staging buffer, one async copy; returns (device views, host views)."""
+    sizes = [meta[f].shape[0] for f in _FIELDS]
+    # each array starts on a 16-byte boundary
+    starts, total = [], 0
+    for n in sizes:
+        starts.append(total)
+        total += (n + 3) // 4 * 4
+    use_gpu = torch.device(device).type == "cuda"
+    staging = torch.empty((max(total, 4),), dtype=torch.int32, pin_memory=use_gpu)
+    host_np = staging.numpy()
+    for f, s, n in zip(_FIELDS, starts, sizes):
+        host_np[s: s + n] = meta[f]
+    dev = staging.to(device, non_blocking=True) if use_gpu else staging
+    dev_views = {f: dev[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
+    host_views = {f: staging[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
+    return dev_views, host_views
+
+
+@dataclass
+class FlashForwardCtx(PagedForwardCtx):
+    indptr: torch.Tensor
+    kv_page_indices: torch.Tensor
+    kv_page_indptr: torch.Tensor
+    kv_last_page_lens: torch.Tensor
+    host: Dict[str, torch.Tensor] = field(default_factory=dict, repr=False)
+
+    @classmethod
+    def init_paged_forward_ctx(cls, task_datas: List[TaskData],
+                               kvcaches: List[PagedKVCache[GpuPagePool]], **extra):
+        pool = kvcaches[0].pool
+        dev, host = upload_metadata(build_host_metadata(task_datas, kvcaches), pool.main_device)
+        return cls(bsz=len(task_datas), seqlens=dev["seqlens"], layer_id=0, page_pool=pool,
+                   offsets=dev["offsets"], indptr=dev["indptr"],
+                   kv_page_indices=dev["kv_page_indices"], kv_page_indptr=dev["kv_page_indptr"],
+                   kv_last_page_lens=dev["kv_last_page_lens"], host=host, **extra)
+
+
+@dataclass
+class FlashDecodeCtx(FlashForwardCtx):
+    decode_wrapper: BatchDecodeWithPagedKVCacheWrapper = None   # type: ignore[assignment]
+
+    @classmethod
+    def init_paged_decode_ctx(cls, task_datas: List[TaskData],
+                              kvcaches: List[PagedKVCache[GpuPagePool]],
+                              wrapper: BatchDecodeWithPagedKVCacheWrapper) -> "FlashDecodeCtx":
+        return cls.init_paged_forward_ctx(task_datas, kvcaches, decode_wrapper=wrapper)
+
+
+@dataclass
+class FlashPrefillCtx(FlashForwardCtx):
+    prefill_wrapper: BatchPrefillWithPagedKVCacheWrapper = None   # type: ignore[assignment]
+
+    @classmethod
+    def init_paged_prefill_ctx(cls, task_datas: List[TaskData],
+                               kvcaches: List[PagedKVCache[GpuPagePool]],
+                               wrapper: BatchPrefillWithPagedKVCacheWrapper) -> "FlashPrefillCtx":
+        return cls.init_paged_forward_ctx(task_datas, kvcaches, prefill_wrapper=wrapper)

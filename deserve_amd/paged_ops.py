@@ -1,0 +1,177 @@
+"""Operators that replace the reference's FlashInfer call sites
+(deserve_worker/model/layer/attention.py:166-192 and
+deserve_worker/execution/exec.py:20-22,184-192,227-236), with the same names,
+argument order and begin_forward/forward/end_forward protocol, implemented by the
+gfx950 kernels behind the C ABI.
+
+All tensors are torch tensors on the GPU; work is enqueued on the current torch
+stream.  ``pages`` is one layer of the pool: (num_pages, 2, page_size, Hkv, D).
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from deserve_amd import _lib
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        raise ValueError(f"index tensors must be int32, got {t.dtype}")
+    return t.contiguous()
+
+
+def append_paged_kv_cache(append_key: torch.Tensor, append_value: torch.Tensor,
+                          append_indptr: torch.Tensor, paged_kv_data: torch.Tensor,
+                          kv_indices: torch.Tensor, kv_indptr: torch.Tensor,
+                          kv_last_page_len: torch.Tensor) -> None:
+    """In place on ``paged_kv_data``: the n_b new tokens of request b become the
+    last n_b positions of its kv_len_b = (npages_b - 1) * P + last_b tokens."""
+    if paged_kv_data.dim() != 5 or paged_kv_data.shape[1] != 2 or not paged_kv_data.is_contiguous():
+        raise ValueError("paged_kv_data must be a contiguous (num_pages, 2, P, Hkv, D) tensor")
+    _, _, P, Hkv, D = paged_kv_data.shape
+    k, v = append_key.contiguous(), append_value.contiguous()
+    if k.shape != v.shape or tuple(k.shape[1:]) != (Hkv, D) or k.dtype != paged_kv_data.dtype \
+            or v.dtype != paged_kv_data.dtype:
+        raise ValueError("append_key/append_value must be (nnz, Hkv, D) of the pool's dtype")
+    rc = _lib.lib().dskv_append_paged_kv(
+        paged_kv_data.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(append_indptr).data_ptr(),
+        _i32(kv_indices).data_ptr(), _i32(kv_indptr).data_ptr(), _i32(kv_last_page_len).data_ptr(),
+        append_indptr.shape[0] - 1, k.shape[0], P, Hkv, D, k.element_size(), _lib.current_stream())
+    _lib.check(rc, "append_paged_kv_cache")
+
+
+def apply_rope(q: torch.Tensor, k: torch.Tensor, indptr: torch.Tensor, offsets: torch.Tensor,
+               interleave: bool = False, rope_scale: float = 1.0,
+               rope_theta: float = 1e4) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Rotary embedding of ragged q (nnz, Hq, D) / k (nnz, Hkv, D); returns new
+    tensors.  Only the adjacent-pair convention (interleave=True) that the
+    reference uses is implemented."""
+    if not interleave or rope_scale != 1.0:
+        raise ValueError("apply_rope: only interleave=True, rope_scale=1 is implemented")
+    q, k = q.contiguous(), k.contiguous()
+    q_out, k_out = torch.empty_like(q), torch.empty_like(k)
+    rc = _lib.lib().dskv_apply_rope(
+        q_out.data_ptr(), k_out.data_ptr(), q.data_ptr(), k.data_ptr(), _i32(indptr).data_ptr(),
+        _i32(offsets).data_ptr(), indptr.shape[0] - 1, q.shape[0], q.shape[1], k.shape[1],
+        q.shape[2], float(rope_theta), _lib.dtype_code(q.dtype), _lib.current_stream())
+    _lib.check(rc, "apply_rope")
+    return q_out, k_out
+
+
+class _PagedWrapper:
+    def __init__(self, workspace_buffer: torch.Tensor, kv_layout: str = "NHD") -> None:
+        if kv_layout != "NHD":
+            raise ValueError("only the NHD page layout is implemented")
+        self._workspace = workspace_buffer
+        self._planned = False
+
+    def _shape_args(self, num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> None:
+        self._hq, self._hkv, self._d, self._p = num_qo_heads, num_kv_heads, head_dim, page_size
+
+    @staticmethod
+    def _host(t: torch.Tensor, host: Optional[torch.Tensor]) -> torch.Tensor:
+        """Host copy of a small index tensor (synchronises only if none was given)."""
+        src = host if host is not None else t.cpu()
+        return src.to(torch.int32).contiguous()
+
+    def end_forward(self) -> None:
+        self._planned = False
+
+
+class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
+    """begin_forward plans the split-KV work list on the host and uploads it once;
+    forward (once per layer) launches the attention and merge kernels."""
+
+    def begin_forward(self, indptr: torch.Tensor, indices: torch.Tensor,
+                      last_page_len: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
+                      head_dim: int, page_size: int, *, indptr_host: Optional[torch.Tensor] = None,
+                      last_page_len_host: Optional[torch.Tensor] = None,
+                      target_items: int = 0, **_ignored) -> None:
+        self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
+        self._indptr, self._indices = _i32(indptr), _i32(indices)
+        h_indptr = self._host(indptr, indptr_host)
+        h_last = self._host(last_page_len, last_page_len_host)
+        batch = h_indptr.shape[0] - 1
+        L = _lib.lib()
+        total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
+        cap = L.dskv_decode_plan_bound(batch, total_tokens)
+        plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
+        n_items, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+        rc = L.dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, page_size,
+                                num_qo_heads, num_kv_heads, head_dim, target_items,
+                                plan.data_ptr(), cap, ctypes.byref(n_items), ctypes.byref(words),
+                                ctypes.byref(ws))
+        _lib.check(rc, "decode begin_forward")
+        if ws.value > self._workspace.numel() * self._workspace.element_size():
+            raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
+        self._batch, self._n_items = batch, n_items.value
+        self._plan_host = plan                       # keep alive until the upload has run
+        self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
+        self._planned = True
+
+    def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,
+                sm_scale: Optional[float] = None, **_ignored) -> torch.Tensor:
+        if not self._planned:
+            raise RuntimeError("decode forward called before begin_forward")
+        q = q.contiguous()
+        if tuple(q.shape) != (self._batch, self._hq, self._d):
+            raise ValueError(f"q must be ({self._batch}, {self._hq}, {self._d}), got {tuple(q.shape)}")
+        if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != q.dtype:
+            raise ValueError("paged_kv_data must be contiguous and of q's dtype")
+        out = torch.empty_like(q)
+        scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
+        rc = _lib.lib().dskv_decode_attn(
+            out.data_ptr(), q.data_ptr(), paged_kv_data.data_ptr(), self._indices.data_ptr(),
+            self._indptr.data_ptr(), self._plan.data_ptr(), self._n_items,
+            self._workspace.data_ptr(), self._workspace.numel() * self._workspace.element_size(),
+            self._batch, self._hq, self._hkv, self._d, self._p, scale, _lib.dtype_code(q.dtype),
+            _lib.current_stream())
+        _lib.check(rc, "decode forward")
+        return out
+
+
+class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
+    def begin_forward(self, qo_indptr: torch.Tensor, paged_kv_indptr: torch.Tensor,
+                      paged_kv_indices: torch.Tensor, paged_kv_last_page_len: torch.Tensor,
+                      num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int, *,
+                      qo_indptr_host: Optional[torch.Tensor] = None, **_ignored) -> None:
+        self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
+        self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
+        self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
+        h_qo = self._host(qo_indptr, qo_indptr_host)
+        batch = h_qo.shape[0] - 1
+        nnz = int(h_qo[-1]) if batch > 0 else 0
+        L = _lib.lib()
+        cap = L.dskv_prefill_plan_bound(batch, nnz)
+        tiles = torch.empty((max(cap, 2),), dtype=torch.int32, pin_memory=True)
+        n_tiles = ctypes.c_int32()
+        rc = L.dskv_prefill_plan(h_qo.data_ptr(), batch, num_qo_heads, num_kv_heads,
+                                 tiles.data_ptr(), cap, ctypes.byref(n_tiles))
+        _lib.check(rc, "prefill begin_forward")
+        self._batch, self._nnz, self._n_tiles = batch, nnz, n_tiles.value
+        self._tiles_host = tiles
+        self._tiles = tiles[: max(2 * n_tiles.value, 2)].to(paged_kv_indices.device, non_blocking=True)
+        self._planned = True
+
+    def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor, causal: bool = True,
+                sm_scale: Optional[float] = None, **_ignored) -> torch.Tensor:
+        if not self._planned:
+            raise RuntimeError("prefill forward called before begin_forward")
+        q = q.contiguous()
+        if tuple(q.shape) != (self._nnz, self._hq, self._d):
+            raise ValueError(f"q must be ({self._nnz}, {self._hq}, {self._d}), got {tuple(q.shape)}")
+        if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != q.dtype:
+            raise ValueError("paged_kv_data must be contiguous and of q's dtype")
+        out = torch.empty_like(q)
+        scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
+        rc = _lib.lib().dskv_prefill_attn(
+            out.data_ptr(), q.data_ptr(), self._qo_indptr.data_ptr(), paged_kv_data.data_ptr(),
+            self._indices.data_ptr(), self._indptr.data_ptr(), self._last.data_ptr(),
+            self._tiles.data_ptr(), self._n_tiles, self._batch, self._nnz, self._hq, self._hkv,
+            self._d, self._p, scale, int(causal), _lib.dtype_code(q.dtype), _lib.current_stream())
+        _lib.check(rc, "prefill forward")
+        return out

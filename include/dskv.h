@@ -1,0 +1,182 @@
+/*
+ * dskv - C ABI of the MI355X (gfx950) KV-cache hot path for one DeServe stage.
+ *
+ * Every entry point is enqueue-only on the HIP stream it is given (passed as an
+ * opaque pointer, i.e. a hipStream_t; NULL is the default stream), takes plain
+ * device/host pointers and sizes, never frees caller memory and never throws.
+ * Return value: 0 = ok, < 0 = argument error (DSKV_E_*), > 0 = a hipError_t.
+ * The message of the last failure on the calling thread is dskv_last_error().
+ *
+ * Reference interfaces replaced (paths relative to the reference repository's
+ * deserve_worker/ package) are cited on each declaration.
+ */
+#ifndef DSKV_H
+#define DSKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSKV_E_INVAL (-1)      /* bad argument / unsupported shape */
+#define DSKV_E_NOMEM (-2)      /* caller buffer too small */
+#define DSKV_E_STATE (-3)      /* handle used in the wrong state */
+
+/* element types of K/V/Q storage */
+#define DSKV_F32 0
+#define DSKV_F16 1
+#define DSKV_BF16 2
+
+const char *dskv_last_error(void);
+int dskv_version(void);
+
+/*
+ * KV append.  Replaces the call site model/layer/attention.py:175-183
+ * (flashinfer.append_paged_kv_cache(xk, xv, indptr, pages, kv_page_indices,
+ * kv_page_indptr, kv_last_page_lens)).
+ * pages_layer: (num_pages, 2, page_size, n_kv_heads, head_dim) of one layer.
+ * k, v: (nnz, n_kv_heads, head_dim) contiguous.  All int32 arrays on device.
+ * Token i of request b goes to position kv_len_b - n_b + i of that request.
+ * Pure byte copy: elt_bytes is 2 or 4.
+ */
+int dskv_append_paged_kv(void *pages_layer, const void *k, const void *v,
+                         const int32_t *qo_indptr, const int32_t *kv_page_indices,
+                         const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
+                         int32_t batch, int32_t nnz, int32_t page_size, int32_t n_kv_heads,
+                         int32_t head_dim, int32_t elt_bytes, void *stream);
+
+/*
+ * Page gather / scatter across all layers.  Replace the advanced-index
+ * gather of kvcache/manager.py:37-42 (and page_pool.py:78-79) and the indexed
+ * assignment of kvcache/manager.py:63-73.
+ * pool: base of (n_layers, num_pages, page_bytes) with layer_stride_bytes
+ * between layers; chunk: contiguous (n_layers * n_pages, page_bytes), layer
+ * major then page_ids order.  page_ids: device int32.  row_begin/row_end select
+ * a sub-range of the n_layers*n_pages chunk rows (0, n_layers*n_pages = all);
+ * chunk points at row row_begin.
+ */
+int dskv_gather_pages(void *chunk, const void *pool, const int32_t *page_ids, int32_t n_pages,
+                      int32_t n_layers, int64_t layer_stride_bytes, int64_t page_bytes,
+                      int64_t row_begin, int64_t row_end, void *stream);
+int dskv_scatter_pages(void *pool, const void *chunk, const int32_t *page_ids, int32_t n_pages,
+                       int32_t n_layers, int64_t layer_stride_bytes, int64_t page_bytes,
+                       int64_t row_begin, int64_t row_end, void *stream);
+
+/*
+ * Paged decode attention.  Replaces BatchDecodeWithPagedKVCacheWrapper
+ * begin_forward (execution/exec.py:184-192) = dskv_decode_plan, and
+ * forward (model/layer/attention.py:185) = dskv_decode_attn.
+ *
+ * dskv_decode_plan runs on the host from host copies of the CSR metadata and
+ * fills plan_host (int32 words) with the split-KV work list; the caller copies
+ * it to the device once per step and reuses it for every layer.
+ *   plan_capacity_words: size of plan_host; required size is at most
+ *                        dskv_decode_plan_bound(batch, total_tokens).
+ *   n_items_out:         number of work items (grid size).
+ *   workspace_bytes_out: device scratch dskv_decode_attn needs for partials.
+ * target_items <= 0 lets the planner choose for the whole chip.
+ */
+int64_t dskv_decode_plan_bound(int32_t batch, int64_t total_tokens);
+int dskv_decode_plan(const int32_t *kv_page_indptr_host, const int32_t *kv_last_page_len_host,
+                     int32_t batch, int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
+                     int32_t head_dim, int32_t target_items, int32_t *plan_host,
+                     int64_t plan_capacity_words, int32_t *n_items_out,
+                     int64_t *plan_words_out, int64_t *workspace_bytes_out);
+
+/*
+ * out, q: (batch, n_qo_heads, head_dim) of dtype; pages_layer as for append.
+ * out[b,h] = softmax_j(q[b,h].K_b[j,h/(Hq/Hkv)] * sm_scale) . V_b[j,h/(Hq/Hkv)]
+ * over the kv_len_b tokens fixed at plan time.  fp32 accumulation.
+ */
+int dskv_decode_attn(void *out, const void *q, const void *pages_layer,
+                     const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
+                     const int32_t *plan_dev, int32_t n_items, void *workspace,
+                     int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
+                     int32_t n_kv_heads, int32_t head_dim, int32_t page_size, float sm_scale,
+                     int32_t dtype, void *stream);
+
+/*
+ * Paged prefill attention with the end-aligned causal mask.  Replaces
+ * BatchPrefillWithPagedKVCacheWrapper.forward(q, pages, causal=True)
+ * (model/layer/attention.py:188-192, execution/exec.py:227-236).
+ * q, out: (nnz, n_qo_heads, head_dim); qo_indptr (batch+1) device int32.
+ * Query i of the n_b queries of request b sees kv positions
+ * j <= kv_len_b - n_b + i.  tile_info_dev: (n_tiles, 2) int32 pairs
+ * (request, first query row of the tile within the request) built by
+ * dskv_prefill_plan from the host copy of qo_indptr (needs at most
+ * dskv_prefill_plan_bound(batch, nnz) words); unused (may be NULL) for fp32.
+ */
+int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz);
+int dskv_prefill_plan(const int32_t *qo_indptr_host, int32_t batch, int32_t n_qo_heads,
+                      int32_t n_kv_heads, int32_t *tile_info_host, int64_t capacity_words,
+                      int32_t *n_tiles_out);
+int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const void *pages_layer,
+                      const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
+                      const int32_t *kv_last_page_len, const int32_t *tile_info_dev,
+                      int32_t n_tiles, int32_t batch, int32_t nnz, int32_t n_qo_heads,
+                      int32_t n_kv_heads, int32_t head_dim, int32_t page_size, float sm_scale,
+                      int32_t causal, int32_t dtype, void *stream);
+
+/*
+ * Rotary embedding, adjacent-pair convention.  Replaces the call site
+ * model/layer/attention.py:166-173 (flashinfer.apply_rope(q, k, indptr,
+ * offsets, interleave=True, rope_theta=5e5)); maths as in
+ * model/layer/attention.py:45-72 with the table of execution/exec.py:25-55.
+ * Out of place: q_out/k_out may alias q/k.
+ */
+int dskv_apply_rope(void *q_out, void *k_out, const void *q, const void *k,
+                    const int32_t *qo_indptr, const int32_t *offsets, int32_t batch, int32_t nnz,
+                    int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim, float rope_theta,
+                    int32_t dtype, void *stream);
+
+/*
+ * Bulk swap of one contiguous page slice of every layer.  Replaces
+ * swap.swap(d, h0, h1, s0, s1, interval) (kvcache/swap.cpp:9-57, called from
+ * kvcache/virtual.py:88-95) with the semantics stated by
+ * VirtualPagePool.swap (kvcache/virtual.py:97-113): for every layer, first
+ * copy slice -> host_to + layer*slice_bytes, then host_from + layer*slice_bytes
+ * -> slice.  Layers [0, L/2) go on stream0, the rest on stream1.  Either host
+ * pointer may be NULL to skip that direction.  Host memory must be pinned.
+ */
+int dskv_swap_slice(void *slice_base, int64_t layer_stride_bytes, int64_t slice_bytes,
+                    int32_t n_layers, void *host_to, const void *host_from, void *stream0,
+                    void *stream1);
+
+/*
+ * Scattered-page swap engine (gather-to-staging + one large async copy per
+ * staging chunk, on the engine's own side streams).  Replaces the blocking
+ * per-task copies KVCacheManager.copy_gpu_to_cpu / copy_cpu_to_gpu
+ * (kvcache/manager.py:24-86); host layout (n_layers*n_pages, page_bytes), layer
+ * major then page_ids order.  page_ids is a HOST int32 array (copied at call
+ * time).  after_stream: work already enqueued there is waited for before the
+ * pool is touched.  dskv_swap_wait blocks the host until everything enqueued
+ * on the handle is done; dskv_swap_fence makes `stream` wait for it instead.
+ */
+typedef struct dskv_swap dskv_swap_t;
+int dskv_swap_create(dskv_swap_t **handle, int64_t staging_bytes);
+int dskv_swap_destroy(dskv_swap_t *handle);
+int dskv_swap_out_async(dskv_swap_t *handle, void *host_dst, const void *pool,
+                        const int32_t *page_ids_host, int32_t n_pages, int32_t n_layers,
+                        int64_t layer_stride_bytes, int64_t page_bytes, void *after_stream);
+int dskv_swap_in_async(dskv_swap_t *handle, void *pool, const void *host_src,
+                       const int32_t *page_ids_host, int32_t n_pages, int32_t n_layers,
+                       int64_t layer_stride_bytes, int64_t page_bytes, void *after_stream);
+/*
+ * Scattered-page counterpart of the microbatch exchange swap.swap performs on a
+ * slice (kvcache/swap.cpp:36-56): the named pages go out to host_dst and are then
+ * refilled from host_src (same layout), chunk by chunk, with the D2H and H2D
+ * traffic on separate streams so both directions of the link are busy.  A chunk
+ * is only overwritten after it has been packed for the trip out.
+ * host_dst == host_src leaves the pages unchanged (only the dump is done).
+ */
+int dskv_swap_exchange_async(dskv_swap_t *handle, void *host_dst, const void *host_src, void *pool,
+                             const int32_t *page_ids_host, int32_t n_pages, int32_t n_layers,
+                             int64_t layer_stride_bytes, int64_t page_bytes, void *after_stream);
+int dskv_swap_wait(dskv_swap_t *handle);
+int dskv_swap_fence(dskv_swap_t *handle, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSKV_H */

@@ -1,0 +1,133 @@
+"""The C-ABI library on a box without a GPU: it loads, exports every symbol the
+header declares, validates arguments before touching the device, and its
+host-side planners satisfy their contracts."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from deserve_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "dskv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dskv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol_and_binding_matches_header():
+    lib = _lib.lib()
+    declared = _declared()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in dskv.h but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == declared
+    assert lib.dskv_version() == 1
+
+
+def test_argument_errors_return_negative_codes_without_a_gpu():
+    lib = _lib.lib()
+    assert lib.dskv_append_paged_kv(1, 1, 1, 1, 1, 1, 1, 2, 2, 16, 8, 128, 3, None) == -1
+    assert "elt_bytes" in _lib.last_error()
+    with pytest.raises(ValueError, match="elt_bytes"):
+        _lib.check(-1, "append")
+    assert lib.dskv_append_paged_kv(None, None, None, None, None, None, None, 0, 0, 16, 8, 128, 2, None) == 0
+    assert lib.dskv_append_paged_kv(None, 1, 1, 1, 1, 1, 1, 1, 1, 16, 8, 128, 2, None) == -1
+    assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 100, 0, 8, None) == -1      # page_bytes % 16
+    assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 64, 3, 9, None) == -1       # row range
+    assert lib.dskv_scatter_pages(16, 16, 16, 4, 2, 1024, 64, 0, 0, None) == 0       # empty range
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 3, None, 0, 2, 32, 8, 128, 16, 0.1, 7, None) == -1
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 3, None, 0, 2, 30, 8, 128, 16, 0.1, 2, None) == -1
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 5, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
+    assert "workspace" in _lib.last_error()
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 2, None, 0, 2, 32, 8, 128, 12, 0.1, 2, None) == -1
+    assert "power-of-two" in _lib.last_error()
+    assert lib.dskv_apply_rope(16, 16, 16, 16, 16, 16, 1, 1, 32, 8, 130, 5e5, 2, None) == -1
+    assert lib.dskv_swap_slice(16, 64, 128, 2, 16, 16, None, None) == -1             # stride < slice
+    assert lib.dskv_swap_slice(None, 0, 0, 0, None, None, None, None) == 0
+    assert lib.dskv_swap_wait(None) == -1 and lib.dskv_swap_out_async(None, 1, 1, 1, 1, 1, 64, 64, None) == -1
+    with pytest.raises(RuntimeError):
+        _lib.check(1, "hip")
+
+
+def _plan(lens, P=16, Hq=32, Hkv=8, D=128, target=0):
+    lib = _lib.lib()
+    lens = np.asarray(lens, np.int64)
+    npages = -(-lens // P)
+    indptr = np.concatenate([[0], np.cumsum(npages)]).astype(np.int32)
+    last = np.where(lens > 0, (lens - 1) % P + 1, 0).astype(np.int32)
+    cap = lib.dskv_decode_plan_bound(len(lens), int(npages.sum()) * P)
+    plan = np.zeros(max(cap, 1), np.int32)
+    n, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+    rc = lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, len(lens), P, Hq, Hkv, D, target,
+                              plan.ctypes.data, cap, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+    assert rc == 0, _lib.last_error()
+    items = plan[: n.value * 4].reshape(-1, 4)
+    req = plan[n.value * 4: words.value].reshape(-1, 2)
+    return items, req, ws.value
+
+
+@pytest.mark.parametrize("lens,target", [([512] * 8, 0), ([1, 15, 16, 17, 4096, 300], 0),
+                                         ([32768, 64, 2048], 64), ([5], 0), ([0, 7], 0),
+                                         (list(range(256, 4097, 61)), 1024)])
+def test_decode_plan_covers_every_token_exactly_once(lens, target):
+    items, req, ws = _plan(lens, target=target)
+    assert req.shape[0] == len(lens)
+    covered = {b: [] for b in range(len(lens))}
+    slots = []
+    for b, t0, t1, slot in items:
+        assert 0 <= t0 <= t1 <= lens[b] and t0 % 16 == 0
+        covered[b].append((t0, t1))
+        if slot >= 0:
+            slots.append((slot, b))
+    for b, n in enumerate(lens):
+        spans = sorted(covered[b])
+        assert spans[0][0] == 0 and spans[-1][1] == n
+        assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))            # contiguous, no overlap
+        first, parts = req[b]
+        if len(spans) == 1:
+            assert parts == 0
+        else:
+            assert parts == len(spans)
+            assert sorted(s for s, bb in slots if bb == b) == list(range(first, first + parts))
+    assert sorted(s for s, _ in slots) == list(range(len(slots)))              # dense slot numbering
+    assert ws == len(slots) * 32 * (128 + 2) * 4
+    sizes = [t1 - t0 for _, t0, t1, _ in items]
+    assert sizes == sorted(sizes, reverse=True)                                # longest first
+
+
+def test_decode_plan_rejects_bad_metadata_and_small_buffers():
+    lib = _lib.lib()
+    indptr = np.array([0, 2], np.int32)
+    last = np.array([17], np.int32)
+    n, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+    plan = np.zeros(64, np.int32)
+    args = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 64, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+    assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *args) == -1
+    last[0] = 16
+    assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *args) == 0
+    small = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 3, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+    assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *small) == -2
+
+
+def test_prefill_plan_tiles_cover_all_query_rows():
+    lib = _lib.lib()
+    qo = np.array([0, 512, 512, 519, 520], np.int32)
+    for hq, hkv in [(32, 8), (64, 8), (8, 8), (32, 1)]:
+        cap = lib.dskv_prefill_plan_bound(4, 520)
+        tiles = np.zeros(cap, np.int32)
+        n = ctypes.c_int32()
+        assert lib.dskv_prefill_plan(qo.ctypes.data, 4, hq, hkv, tiles.ctypes.data, cap, ctypes.byref(n)) == 0
+        t = tiles[: 2 * n.value].reshape(-1, 2)
+        group = hq // hkv
+        rows = 2 * (16 // group) if group <= 16 else 1
+        for b in range(4):
+            nb = qo[b + 1] - qo[b]
+            starts = sorted(t[t[:, 0] == b][:, 1].tolist())
+            assert starts == list(range(0, nb, rows))
+    n = ctypes.c_int32()
+    assert lib.dskv_prefill_plan(qo.ctypes.data, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2

@@ -1,0 +1,294 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on a real
+MI355X.  Copy-type operators must be bit-exact; attention must stay within
+2e-2 of the fp32 oracle, measured as max |got - ref| / max |ref| (error relative
+to the output's scale), for 16-bit storage and 1e-4 for fp32 storage."""
+import numpy as np
+import pytest
+import torch
+
+from kvutil import from_torch, make_scenario, max_rel_err, to_torch, torch_dtype
+from oracle import c_oracle
+from oracle import kv_oracle as orc
+
+pytestmark = pytest.mark.gpu
+ATTN_TOL = {"bf16": 2e-2, "f16": 2e-2, "f32": 1e-4}
+
+
+def _dev_i32(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.int32)).cuda()
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+# ------------------------------------------------------------------ append
+@pytest.mark.parametrize("dtype", ["bf16", "f32", "f16"])
+@pytest.mark.parametrize("P", [16, 8])
+def test_append_bit_exact(dtype, P):
+    from deserve_amd.paged_ops import append_paged_kv_cache
+
+    cases = {
+        "decode": dict(kv_lens=[512, 1, 17, 16, 4096, 33, 250, 15], qo_lens=[1] * 8),
+        "chunk": dict(kv_lens=[517, 40, 512, 3, 1029], qo_lens=[512, 40, 7, 3, 0]),
+    }
+    for name, c in cases.items():
+        _announce("append", dtype, P, name)
+        sc = make_scenario(21, P=P, dtype=dtype, **c)
+        want = sc.pages.copy()
+        orc.append_paged_kv(want, sc.k, sc.v, sc.qo_indptr, sc.kv_page_indices, sc.kv_page_indptr,
+                            sc.kv_last_page_lens)
+        pages = to_torch(sc.pages, dtype)
+        append_paged_kv_cache(to_torch(sc.k, dtype), to_torch(sc.v, dtype), _dev_i32(sc.qo_indptr),
+                              pages, _dev_i32(sc.kv_page_indices), _dev_i32(sc.kv_page_indptr),
+                              _dev_i32(sc.kv_last_page_lens))
+        torch.cuda.synchronize()
+        got = from_torch(pages, dtype)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))     # includes untouched bytes
+
+
+def test_append_rejects_wrong_shapes():
+    from deserve_amd.paged_ops import append_paged_kv_cache
+
+    pages = torch.zeros((4, 2, 16, 8, 128), dtype=torch.bfloat16, device="cuda")
+    k = torch.zeros((1, 8, 64), dtype=torch.bfloat16, device="cuda")
+    i = torch.zeros(2, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        append_paged_kv_cache(k, k, i, pages, i, i, i)
+    with pytest.raises(ValueError):
+        append_paged_kv_cache(k, k, i.long(), pages[:, :, :, :, :64].contiguous(), i, i, i)
+
+
+# ------------------------------------------------------------------ gather / scatter
+@pytest.mark.parametrize("dtype,P", [("bf16", 16), ("f32", 16), ("f16", 8)])
+def test_gather_scatter_bit_exact(dtype, P):
+    from deserve_amd.kvcache import _native
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+
+    _announce("gather/scatter", dtype, P)
+    rng = np.random.default_rng(5)
+    L, n = 3, 40
+    pool = GpuPagePool(L, n, P, torch.device("cuda"), torch_dtype(dtype))
+    raw = rng.integers(0, 256, size=pool.pages.numel() * pool.pages.element_size(), dtype=np.uint8)
+    pool.pages.view(torch.uint8).view(-1).copy_(torch.from_numpy(raw))
+    host = from_torch(pool.pages, dtype)
+    for ids in ([7, 0, 39, 3, 21], list(range(40)), [], [5]):
+        ids_t = torch.tensor(ids, dtype=torch.int32)
+        got = from_torch(pool.retrieve(ids_t), dtype)
+        want = orc.gather_pages(host, ids)
+        assert got.shape == (L, len(ids)) + host.shape[2:]
+        assert np.array_equal(got.reshape(want.shape), want)
+        if ids:
+            assert np.array_equal(c_oracle.gather(host, ids), want)
+    ids = [9, 2, 30]
+    chunk = rng.integers(0, 2**16, size=(L * 3,) + host.shape[2:]).astype(host.dtype) \
+        if dtype != "f32" else rng.standard_normal((L * 3,) + host.shape[2:]).astype(np.float32)
+    want = host.copy()
+    orc.scatter_pages(want, ids, chunk)
+    _native.scatter_pages(pool, torch.tensor(ids, dtype=torch.int32), to_torch(chunk, dtype))
+    torch.cuda.synchronize()
+    assert np.array_equal(from_torch(pool.pages, dtype).view(np.uint8), want.view(np.uint8))
+
+
+# ------------------------------------------------------------------ decode attention
+def _run_decode(sc, target_items=0):
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    w = BatchDecodeWithPagedKVCacheWrapper(ws)
+    w.begin_forward(_dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                    _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P,
+                    target_items=target_items)
+    out = w.forward(to_torch(sc.q, sc.dtype), to_torch(sc.pages, sc.dtype))
+    w.end_forward()
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy(), w._n_items
+
+
+DECODE_CASES = [
+    # (name, kv_lens, P, Hq, Hkv, D, dtype, target_items)
+    ("tiny", [1, 2, 15, 16, 17, 31, 32, 33], 16, 32, 8, 128, "bf16", 0),
+    ("split", [4096, 700, 257, 3000], 16, 32, 8, 128, "bf16", 64),
+    ("nosplit", [4096, 700, 257, 3000], 16, 32, 8, 128, "bf16", 1),
+    ("group8", [1000, 64, 2049, 5], 16, 64, 8, 128, "bf16", 32),
+    ("f16", [1000, 64, 333], 16, 32, 8, 128, "f16", 16),
+    ("page8", [1000, 64, 333, 7, 8, 9], 8, 32, 8, 128, "bf16", 16),
+    ("page4", [100, 3, 19], 4, 32, 8, 128, "f16", 4),
+    ("page32", [1000, 31, 33, 64], 32, 32, 8, 128, "bf16", 16),
+    ("mha", [300, 40], 16, 8, 8, 128, "bf16", 0),
+    ("group16", [300, 40], 16, 32, 2, 128, "bf16", 8),
+    ("kv4", [300, 40, 1], 16, 16, 4, 128, "bf16", 0),
+    ("f32", [512, 100, 1, 33], 16, 32, 8, 128, "f32", 8),
+    ("f32_d64", [200, 17], 8, 8, 2, 64, "f32", 0),
+    ("bf16_d64_generic", [200, 17], 16, 8, 2, 64, "bf16", 4),
+    ("empty_request", [0, 50], 16, 32, 8, 128, "bf16", 0),
+]
+
+
+@pytest.mark.parametrize("case", DECODE_CASES, ids=[c[0] for c in DECODE_CASES])
+def test_decode_attention_matches_oracle(case):
+    name, lens, P, Hq, Hkv, D, dtype, target = case
+    _announce("decode", *case)
+    sc = make_scenario(31, kv_lens=lens, qo_lens=[1] * len(lens), P=P, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype)
+    got, n_items = _run_decode(sc, target)
+    want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                sc.kv_last_page_lens, dtype)
+    live = np.asarray(lens) > 0
+    assert np.isfinite(got).all()
+    assert max_rel_err(got[live], want[live]) <= ATTN_TOL[dtype]
+    assert not got[~live].any()                       # a request without tokens yields zeros
+    if name == "split":
+        assert n_items > len(lens)
+    if name == "nosplit":
+        assert n_items == len(lens)
+
+
+def test_decode_attention_ignores_garbage_beyond_kv_len():
+    """Slots past the last valid token of the last page hold NaN/Inf bit patterns."""
+    _announce("decode garbage tail")
+    sc = make_scenario(32, kv_lens=[5, 33, 100], qo_lens=[1, 1, 1], dtype="bf16")
+    clean, _ = _run_decode(sc)
+    for b in range(3):
+        last_page = sc.kv_page_indices[sc.kv_page_indptr[b + 1] - 1]
+        sc.pages[last_page, :, int(sc.kv_last_page_lens[b]):] = 0x7FC0      # NaN
+    spare = np.setdiff1d(np.arange(sc.num_pages), sc.kv_page_indices)
+    sc.pages[spare] = 0x7F80                                              # +Inf in unowned pages
+    dirty, _ = _run_decode(sc)
+    assert np.array_equal(clean, dirty)
+
+
+def test_decode_attention_closed_forms_on_gpu():
+    _announce("decode closed forms")
+    sc = make_scenario(33, kv_lens=[1, 40], qo_lens=[1, 1], dtype="bf16")
+    sc.pages[sc.kv_page_indices[sc.kv_page_indptr[1]: sc.kv_page_indptr[2]], 0] = 0x3E80   # all keys 0.25
+    got, _ = _run_decode(sc)
+    pf = orc.to_f32(sc.pages, "bf16")
+    page0 = sc.kv_page_indices[0]
+    assert max_rel_err(got[0], np.repeat(pf[page0, 1, 0], 4, axis=0)) < 1e-2      # kv_len 1 -> V row
+    ids = sc.kv_page_indices[sc.kv_page_indptr[1]: sc.kv_page_indptr[2]]
+    v = pf[ids, 1].reshape(-1, 8, 128)[:40].mean(axis=0)
+    assert max_rel_err(got[1], np.repeat(v, 4, axis=0)) < 2e-2                    # equal keys -> mean V
+
+
+def test_decode_wrapper_protocol_errors():
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    q = torch.zeros((1, 32, 128), dtype=torch.bfloat16, device="cuda")
+    pages = torch.zeros((4, 2, 16, 8, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="begin_forward"):
+        w.forward(q, pages)
+    w.begin_forward(_dev_i32([0, 1]), _dev_i32([2]), _dev_i32([3]), 32, 8, 128, 16)
+    with pytest.raises(ValueError):
+        w.forward(q[:, :16], pages)
+    w.forward(q, pages)
+    w.end_forward()
+    with pytest.raises(RuntimeError):
+        w.forward(q, pages)
+    small = BatchDecodeWithPagedKVCacheWrapper(torch.empty(1024, dtype=torch.uint8, device="cuda"))
+    with pytest.raises(RuntimeError, match="workspace"):
+        small.begin_forward(_dev_i32([0, 256]), _dev_i32(list(range(256))), _dev_i32([16]), 32, 8,
+                            128, 16, target_items=8)
+    with pytest.raises(ValueError):
+        w.begin_forward(_dev_i32([0, 1]), _dev_i32([2]), _dev_i32([17]), 32, 8, 128, 16)
+
+
+# ------------------------------------------------------------------ prefill attention
+PREFILL_CASES = [
+    ("chunks", [517, 40, 512, 3], [512, 40, 7, 3], 16, 32, 8, 128, "bf16"),
+    ("ragged_prior", [1500, 16, 33, 700], [100, 16, 1, 65], 16, 32, 8, 128, "bf16"),
+    ("group8", [300, 77], [128, 77], 16, 64, 8, 128, "bf16"),
+    ("f16_page8", [300, 77, 9], [50, 77, 1], 8, 32, 8, 128, "f16"),
+    ("mha", [100, 20], [30, 20], 16, 8, 8, 128, "bf16"),
+    ("f32", [60, 20], [30, 20], 16, 8, 2, 128, "f32"),
+    ("empty_chunk", [60, 20, 40], [30, 0, 5], 16, 32, 8, 128, "bf16"),
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_CASES, ids=[c[0] for c in PREFILL_CASES])
+def test_prefill_attention_matches_oracle(case):
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+
+    name, kv, qo, P, Hq, Hkv, D, dtype = case
+    _announce("prefill", *case)
+    sc = make_scenario(41, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                    _dev_i32(sc.kv_last_page_lens), Hq, Hkv, D, P)
+    for causal in (True, False):
+        out = w.forward(to_torch(sc.q, dtype), to_torch(sc.pages, dtype), causal=causal)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
+                                     sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
+        assert np.isfinite(got).all()
+        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (name, causal)
+    w.end_forward()
+
+
+def test_prefill_with_one_query_equals_decode():
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+
+    _announce("prefill n=1 vs decode")
+    sc = make_scenario(42, kv_lens=[700, 33, 16], qo_lens=[1, 1, 1], dtype="bf16")
+    dec, _ = _run_decode(sc, target_items=1)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                    _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P)
+    pre = w.forward(to_torch(sc.q, "bf16"), to_torch(sc.pages, "bf16")).float().cpu().numpy()
+    assert max_rel_err(pre, dec) < 1e-2
+
+
+# ------------------------------------------------------------------ rope
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+def test_rope_matches_oracle(dtype):
+    from deserve_amd.paged_ops import apply_rope
+
+    _announce("rope", dtype)
+    rng = np.random.default_rng(51)
+    indptr = np.array([0, 1, 6, 6, 40], np.int32)
+    offsets = np.array([511, 0, 3, 4000], np.int32)
+    q = rng.standard_normal((40, 32, 128)).astype(np.float32)
+    k = rng.standard_normal((40, 8, 128)).astype(np.float32)
+    from kvutil import to_storage
+    qs, ks = to_storage(q, dtype), to_storage(k, dtype)
+    q_out, k_out = apply_rope(to_torch(qs, dtype), to_torch(ks, dtype), _dev_i32(indptr),
+                              _dev_i32(offsets), interleave=True, rope_theta=500000.0)
+    torch.cuda.synchronize()
+    want_q = orc.rope_interleaved(orc.to_f32(qs, dtype), indptr, offsets)
+    want_k = orc.rope_interleaved(orc.to_f32(ks, dtype), indptr, offsets)
+    tol = {"f32": 2e-3, "bf16": 1.2e-2, "f16": 3e-3}[dtype]   # fp32: angle of 4000 rad in fp32
+    assert np.abs(q_out.float().cpu().numpy() - want_q).max() <= tol * np.abs(want_q).max()
+    assert np.abs(k_out.float().cpu().numpy() - want_k).max() <= tol * np.abs(want_k).max()
+    with pytest.raises(ValueError):
+        apply_rope(to_torch(qs, dtype), to_torch(ks, dtype), _dev_i32(indptr), _dev_i32(offsets))
+
+
+# ------------------------------------------------------------------ config 1 of the baseline, exactly
+def test_baseline_config1_fp32_append_then_decode():
+    """8 sequences, context 512 after the append, 256-page pool in a seeded random
+    permutation, fp32, 32 q heads / 8 kv heads / head_dim 128, page size 16."""
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper, append_paged_kv_cache
+
+    _announce("config1")
+    sc = make_scenario(1, kv_lens=[512] * 8, qo_lens=[1] * 8, dtype="f32", spare_pages=0)
+    assert sc.num_pages == 256
+    want_pages = sc.pages.copy()
+    orc.append_paged_kv(want_pages, sc.k, sc.v, sc.qo_indptr, sc.kv_page_indices, sc.kv_page_indptr,
+                        sc.kv_last_page_lens)
+    want = orc.decode_attention(sc.q, want_pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                sc.kv_last_page_lens, "f32")
+    pages = to_torch(sc.pages, "f32")
+    args = [_dev_i32(x) for x in (sc.qo_indptr, sc.kv_page_indices, sc.kv_page_indptr, sc.kv_last_page_lens)]
+    append_paged_kv_cache(to_torch(sc.k, "f32"), to_torch(sc.v, "f32"), args[0], pages, args[1], args[2], args[3])
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(16 << 20, dtype=torch.uint8, device="cuda"))
+    w.begin_forward(args[2], args[1], args[3], 32, 8, 128, 16)
+    got = w.forward(to_torch(sc.q, "f32"), pages).cpu().numpy()
+    assert np.array_equal(from_torch(pages, "f32"), want_pages)
+    assert max_rel_err(got, want) <= 1e-4
+    # the same problem in bf16 storage stays within the 16-bit tolerance of the fp32 answer
+    scb = make_scenario(1, kv_lens=[512] * 8, qo_lens=[1] * 8, dtype="bf16", spare_pages=0)
+    got_b, _ = _run_decode(scb)
+    want_b = orc.decode_attention(scb.q, scb.pages, scb.kv_page_indices, scb.kv_page_indptr,
+                                  scb.kv_last_page_lens, "bf16")
+    assert max_rel_err(got_b, want_b) <= 2e-2
