@@ -14,35 +14,29 @@ template <int DT> struct Chunk;   // 16 bytes <-> fp32 lanes
 template <> struct Chunk<DSKV_F32> {
     static constexpr int kElems = 4;
     static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) f[i] = __builtin_bit_cast(float, raw[i]);
+        const f32x4 v = __builtin_bit_cast(f32x4, raw);
+        f[0] = v.x;
+        f[1] = v.y;
+        f[2] = v.z;
+        f[3] = v.w;
     }
     static __device__ __forceinline__ u32x4 pack(const float *f) {
-        u32x4 r;
-#pragma unroll
-        for (int i = 0; i < 4; i++) r[i] = __builtin_bit_cast(uint32_t, f[i]);
-        return r;
+        const f32x4 v = {f[0], f[1], f[2], f[3]};
+        return __builtin_bit_cast(u32x4, v);
     }
 };
 template <> struct Chunk<DSKV_F16> {
     static constexpr int kElems = 8;
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    typedef float f8 __attribute__((ext_vector_type(8)));
     static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            h2 p = __builtin_bit_cast(h2, raw[i]);
-            f[2 * i] = (float)p[0];
-            f[2 * i + 1] = (float)p[1];
-        }
+        const f8 v = __builtin_convertvector(__builtin_bit_cast(h8, raw), f8);
+        f[0] = v.s0; f[1] = v.s1; f[2] = v.s2; f[3] = v.s3;
+        f[4] = v.s4; f[5] = v.s5; f[6] = v.s6; f[7] = v.s7;
     }
     static __device__ __forceinline__ u32x4 pack(const float *f) {
-        u32x4 r;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            h2 p = {(_Float16)f[2 * i], (_Float16)f[2 * i + 1]};
-            r[i] = __builtin_bit_cast(uint32_t, p);
-        }
-        return r;
+        const f8 v = {f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]};
+        return __builtin_bit_cast(u32x4, __builtin_convertvector(v, h8));
     }
 };
 template <> struct Chunk<DSKV_BF16> {
