@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache hot path of one Llama-3-8B pipeline stage on one MI355X.
+
+Workload (baseline configuration 2): 16 layers, bf16, GQA 32 q / 8 kv heads,
+head_dim 128, page size 16, decode batch of 64 sequences with context lengths
+seeded uniform in [256, 4096], pages scattered over the pool by a seeded
+permutation, K/V ~ N(0, 1).  One step = build the step's metadata and attention
+plan on the host, then per layer: append 1 token per sequence and run paged
+decode attention.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is the algorithmic KV bytes one step moves
+(append + decode attention, every layer) divided by the wall time of a step.
+`roofline` is for the dominant kernel (the split-KV decode attention pass),
+timed with events on the launch stream inside the timed region.
+`cpu_baseline` times the scalar C port of the same maths (OpenMP over
+request x head) on a bounded sample, on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seed", type=int, default=2)
+    ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
+    ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-events", action="store_true",
+                    help="do not bracket the attention pass with events (pure step timing)")
+    return ap.parse_args()
+
+
+def attention_bytes_per_layer(kv_lens, n_pages_total, batch, hq, d, e, kv_token_bytes) -> int:
+    """sum_b kv_len_b * 2*Hkv*D*e  +  Q read and O write  +  block-table entries."""
+    return int(kv_lens.sum()) * kv_token_bytes + 2 * batch * hq * d * e + 4 * int(n_pages_total)
+
+
+def append_bytes_per_layer(nnz, batch, n_pages_total, kv_token_bytes) -> int:
+    """read the new K, V rows and write them, plus the int32 metadata."""
+    return 2 * nnz * kv_token_bytes + 4 * (3 * batch + 2 + int(n_pages_total))
+
+
+def cpu_baseline(wl, meta, sample_requests: int):
+    """Scalar C port (oracle/kv_oracle.c) of append + decode attention for ONE layer of
+    the first `sample_requests` requests of the same workload, on the host cores."""
+    import numpy as np
+
+    from oracle import c_oracle
+
+    c_oracle.load()
+    B = sample_requests
+    indptr = meta["kv_page_indptr"][: B + 1].astype(np.int32)
+    ids = meta["kv_page_indices"][: indptr[-1]].astype(np.int32)
+    last = meta["kv_last_page_lens"][:B].astype(np.int32)
+    # compact copy of the sample's pages (bf16 bits) so the host holds MBs, not the pool
+    import torch
+
+    sel = torch.from_numpy(ids.astype(np.int64)).to(wl.pool.pages.device)
+    pages = wl.pool.pages[0].index_select(0, sel).cpu().view(torch.int16).numpy().view(np.uint16)
+    local_ids = np.arange(len(ids), dtype=np.int32)
+    as_bits = lambda t: t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    q, k, v = as_bits(wl.q[0, :B]), as_bits(wl.k[0, :B]), as_bits(wl.v[0, :B])
+    qo = np.arange(B + 1, dtype=np.int32)
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    P = wl.args.page_size
+    kv_lens = (np.diff(indptr) - 1) * P + last
+    tok_bytes = wl.kv_bytes_per_token()
+    nbytes = attention_bytes_per_layer(kv_lens, len(ids), B, wl.args.n_heads, 128, 2, tok_bytes) + \
+        append_bytes_per_layer(B, B, len(ids), tok_bytes)
+    times = []
+    t_end = time.time() + 20.0
+    while len(times) < 3 or (time.time() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        c_oracle.append(pages, k, v, qo, local_ids, indptr, last, "bf16")
+        c_oracle.decode_attn(q, pages, local_ids, indptr, last, "bf16")
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"1 of {wl.args.n_layers} layers, first {B} of {wl.batch} sequences "
+                      f"({int(kv_lens.sum())} kv tokens), median of {len(times)} runs, "
+                      f"{med * 1e3:.1f} ms each, scalar C + OpenMP"}
+
+
+def main() -> int:
+    a = parse_args()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU: --gpus {a.gpus} is not supported in this build "
+              "(the path has no cross-GPU exchange; see DESIGN.md on sharding)", file=sys.stderr)
+        return 2
+    import numpy as np
+    import torch
+
+    from deserve_amd import _lib
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.paged_ops import append_paged_kv_cache, apply_rope
+    from deserve_amd.synthetic import config2_context_lengths, make_decode_workload
+
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    torch.cuda.set_device(0)
+    L, Hq, Hkv, D, P = 16, 32, 8, 128, 16
+    total_steps = a.steps + a.warmup
+    ctx = config2_context_lengths(a.seed)
+    wl = make_decode_workload("cfg2", ctx, L, Hq, Hkv, D, P, torch.bfloat16,
+                              headroom_tokens=total_steps + 8, seed=a.seed, use_rope=a.rope)
+    decode_wrapper, _ = get_wrappers(wl.pool.main_device)
+    e = wl.pool.pages.element_size()
+    tok_bytes = wl.kv_bytes_per_token()
+    torch.cuda.synchronize()
+
+    ev_pairs = []          # (start, end) events around the split-KV attention pass
+    step_bytes = []
+    attn_bytes_layer = []
+
+    def one_step(timed: bool):
+        """prepare (metadata + plan, one upload each) then L x (append, attention)."""
+        c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, decode_wrapper)
+        decode_wrapper.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
+                                     last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
+                                     num_kv_heads=Hkv, head_dim=D, page_size=P,
+                                     indptr_host=c.host["kv_page_indptr"],
+                                     last_page_len_host=c.host["kv_last_page_lens"],
+                                     target_workgroups=a.workgroups)
+        for layer in range(L):
+            q, k, v = wl.q[layer], wl.k[layer], wl.v[layer]
+            if a.rope:
+                q, k = apply_rope(q, k, c.indptr, c.offsets, interleave=True, rope_theta=5e5)
+            pages = wl.pool.get_layered_pages(layer)
+            append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
+                                  c.kv_last_page_lens)
+            if timed and not a.no_kernel_events:
+                s, t = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                out = decode_wrapper.forward(q, pages, phases=1)
+                t.record()
+                decode_wrapper.forward(q, pages, phases=2, out=out)
+                ev_pairs.append((s, t))
+            else:
+                decode_wrapper.forward(q, pages)
+        decode_wrapper.end_forward()
+        if timed:
+            kv_lens = np.array([t.start_pos + 1 for t in wl.tasks], dtype=np.int64)
+            n_pages = int(c.host["kv_page_indptr"][-1])
+            ab = attention_bytes_per_layer(kv_lens, n_pages, wl.batch, Hq, D, e, tok_bytes)
+            attn_bytes_layer.append(ab)
+            step_bytes.append(L * (ab + append_bytes_per_layer(wl.batch, wl.batch, n_pages, tok_bytes)))
+        for t in wl.tasks:
+            t.step()
+        return c
+
+    last_ctx = None
+    for _ in range(a.warmup):
+        last_ctx = one_step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        last_ctx = one_step(True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    ms_per_step = elapsed / a.steps * 1e3
+    value = sum(step_bytes) / elapsed / 1e9
+    out = {
+        "metric": "paged decode-attn HBM GB/s", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE.json configs[1]: Llama-3-8B stage, 16 layers, bf16, GQA 32q/8kv, "
+                               "head_dim 128, page 16, decode batch 64, ctx U[256,4096], scattered pages; "
+                               "step = host plan + 16 x (append 1 token + paged decode attention)"
+                               + (" + RoPE" if a.rope else ""),
+                   "batch": wl.batch, "layers": L, "kv_tokens": int(sum(t.start_pos for t in wl.tasks)),
+                   "work_items": decode_wrapper._n_items, "workgroups": decode_wrapper._n_workgroups, "seed": a.seed},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "stage_tokens_per_s": round(wl.batch / (elapsed / a.steps), 1),
+    }
+    if ev_pairs:
+        times_ms = [s.elapsed_time(t) for s, t in ev_pairs]
+        avg_ms = sum(times_ms) / len(times_ms)
+        achieved = (sum(attn_bytes_layer) / len(attn_bytes_layer)) / (avg_ms * 1e-3) / 1e9
+        traffic = None
+        tfile = os.path.join(ROOT, "profiles", "decode_attn_cfg2_traffic.json")
+        if os.path.exists(tfile):
+            traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
+        out["roofline"] = {"bound": "hbm", "kernel": "decode_attn_mfma_kernel<bf16> (split-KV pass)",
+                           "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                           "avg_launch_us": round(avg_ms * 1e3, 2), "launches": len(times_ms),
+                           "algorithmic_bytes_per_launch": int(sum(attn_bytes_layer) / len(attn_bytes_layer))}
+    if not a.no_cpu_baseline:
+        meta = {n: last_ctx.host[n].numpy() for n in ("kv_page_indices", "kv_page_indptr", "kv_last_page_lens")}
+        out["cpu_baseline"] = cpu_baseline(wl, meta, sample_requests=16)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -25,6 +25,13 @@ constexpr int kOutOfRange = 0x7FFF0000;   // byte offset no page reaches: reads 
 // MFMA row m of a tile holds token (m >> 2) + 4 * (m & 3) of that tile.
 __device__ __forceinline__ int row_to_token(int m) { return (m >> 2) + ((m & 3) << 2); }
 
+// Block tables and work lists never change while a kernel runs.  Reading them
+// through the constant address space tells the compiler so: wave-uniform reads
+// become scalar loads (tracked apart from the vector loads of the K/V stream)
+// even after the kernel has issued stores.
+typedef const __attribute__((address_space(4))) int32_t *const_i32_ptr;
+__device__ __forceinline__ const_i32_ptr as_const(const int32_t *p) { return (const_i32_ptr)p; }
+
 struct TileRegs {
     u32x4 k[4];
     u32x4 v[4];
@@ -33,13 +40,49 @@ struct TileRegs {
 // One request's paged K/V of one layer as seen by one wave (one kv head).
 struct KvView {
     const char *pages;           // layer base: (num_pages, 2, P, Hkv, 128) 16-bit
-    const int32_t *page_ids;     // this request's block-table entries
+    const_i32_ptr page_ids;      // this request's block-table entries
     int page_shift;              // log2(page_size)
     int row_bytes;               // one token, all kv heads
     int half_bytes;              // K half of a page
     long page_bytes;
     int head_off;                // byte offset of this wave's kv head inside a token row
 };
+
+// Loads tile [t, t + 16), which lies inside pool page `page`, of a request whose
+// valid tokens end at t_end.  The page is addressed through a buffer descriptor:
+// rows at or past t_end get an offset outside the page and a tile past the end
+// gets an empty descriptor, so such lanes read zero and generate no memory
+// traffic.  Always issues exactly 8 loads.
+__device__ __forceinline__ void load_kv_tile_in_page(const KvView &kv, long page, int t, int t_end,
+                                                     int g, int c, TileRegs &r)
+{
+    const int k_tok = row_to_token(c);
+    const int slot_off = (t & ((1 << kv.page_shift) - 1)) * kv.row_bytes;
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char *>(kv.pages) + page * kv.page_bytes, 0, t < t_end ? (int)kv.page_bytes : 0,
+        kBufferFlags);
+    const int ko = (t + k_tok < t_end) ? slot_off + k_tok * kv.row_bytes + kv.head_off + g * 16
+                                       : kOutOfRange;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++)
+        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int vo = (t + g + 4 * i < t_end)
+                           ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes + kv.head_off +
+                                 c * 16
+                           : kOutOfRange;
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, 0);
+    }
+}
+
+// Index into the request's block table of the page that holds token t, clamped
+// to the last page the request owns (a tile past the end still names a valid
+// entry; its descriptor is empty anyway).
+__device__ __forceinline__ int page_slot_of(const KvView &kv, int t, int t_end)
+{
+    return min(t >> kv.page_shift, max((t_end - 1) >> kv.page_shift, 0));
+}
 
 // Loads tile [t, t + 16) of a request whose valid tokens end at t_end.  Issued
 // unconditionally (so the count of loads in flight is static); nothing past
@@ -48,36 +91,13 @@ template <bool kPageCoversTile>
 __device__ __forceinline__ void load_kv_tile(const KvView &kv, int t, int t_end, int g, int c,
                                              TileRegs &r)
 {
-    const int k_tok = row_to_token(c);
     if (kPageCoversTile) {
-        // One page holds the whole tile: address it through a buffer descriptor
-        // of that page.  Rows at or past t_end get an offset outside the page
-        // and a tile past the end gets an empty descriptor: such lanes read zero
-        // and generate no memory traffic.
-        const int page_size = 1 << kv.page_shift;
-        const int last_page = max((t_end - 1) >> kv.page_shift, 0);
-        const long page = kv.page_ids[min(t >> kv.page_shift, last_page)];
-        const int slot_off = (t & (page_size - 1)) * kv.row_bytes;
-        __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<char *>(kv.pages) + page * kv.page_bytes, 0,
-            t < t_end ? (int)kv.page_bytes : 0, kBufferFlags);
-        const int ko = (t + k_tok < t_end) ? slot_off + k_tok * kv.row_bytes + kv.head_off + g * 16
-                                           : kOutOfRange;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-            r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int vo = (t + g + 4 * i < t_end)
-                               ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes +
-                                     kv.head_off + c * 16
-                               : kOutOfRange;
-            r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, 0);
-        }
+        load_kv_tile_in_page(kv, kv.page_ids[page_slot_of(kv, t, t_end)], t, t_end, g, c, r);
     } else {
         // Pages smaller than a tile: every lane resolves its own page.  Tokens
         // past the end are clamped to the last valid one; the consumer masks
         // their scores and zeroes their V rows.
+        const int k_tok = row_to_token(c);
         const int page_mask = (1 << kv.page_shift) - 1;
         const int t_last = max(t_end - 1, 0);
         const int tk = min(t + k_tok, t_last);

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
 
     KvView kv;
     kv.pages = pages;
-    kv.page_ids = kv_indices + kv_indptr[b];
+    kv.page_ids = as_const(kv_indices) + kv_indptr[b];
     kv.page_shift = page_shift;
     kv.row_bytes = n_kv_heads * kHeadDim * 2;
     kv.half_bytes = kv.row_bytes << page_shift;

@@ -90,7 +90,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
                       last_page_len: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, *, indptr_host: Optional[torch.Tensor] = None,
                       last_page_len_host: Optional[torch.Tensor] = None,
-                      target_items: int = 0, **_ignored) -> None:
+                      target_workgroups: int = 0, **_ignored) -> None:
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._indptr, self._indices = _i32(indptr), _i32(indices)
         h_indptr = self._host(indptr, indptr_host)
@@ -100,21 +100,24 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
         cap = L.dskv_decode_plan_bound(batch, total_tokens)
         plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
-        n_items, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+        n_items, n_wgs = ctypes.c_int32(), ctypes.c_int32()
+        words, ws = ctypes.c_int64(), ctypes.c_int64()
         rc = L.dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, page_size,
-                                num_qo_heads, num_kv_heads, head_dim, target_items,
-                                plan.data_ptr(), cap, ctypes.byref(n_items), ctypes.byref(words),
-                                ctypes.byref(ws))
+                                num_qo_heads, num_kv_heads, head_dim, target_workgroups,
+                                plan.data_ptr(), cap, ctypes.byref(n_items), ctypes.byref(n_wgs),
+                                ctypes.byref(words), ctypes.byref(ws))
         _lib.check(rc, "decode begin_forward")
         if ws.value > self._workspace.numel() * self._workspace.element_size():
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
-        self._batch, self._n_items = batch, n_items.value
+        self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
         self._plan_host = plan                       # keep alive until the upload has run
         self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
         self._planned = True
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,
-                sm_scale: Optional[float] = None, **_ignored) -> torch.Tensor:
+                sm_scale: Optional[float] = None, *, phases: int = 3,
+                out: Optional[torch.Tensor] = None, **_ignored) -> torch.Tensor:
+        """phases: 1 = split-KV pass only, 2 = merge pass only, 3 = both (default)."""
         if not self._planned:
             raise RuntimeError("decode forward called before begin_forward")
         q = q.contiguous()
@@ -122,14 +125,14 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
             raise ValueError(f"q must be ({self._batch}, {self._hq}, {self._d}), got {tuple(q.shape)}")
         if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != q.dtype:
             raise ValueError("paged_kv_data must be contiguous and of q's dtype")
-        out = torch.empty_like(q)
+        if out is None:
+            out = torch.empty_like(q)
         scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
-        rc = _lib.lib().dskv_decode_attn(
+        rc = _lib.lib().dskv_decode_attn_phases(
             out.data_ptr(), q.data_ptr(), paged_kv_data.data_ptr(), self._indices.data_ptr(),
-            self._indptr.data_ptr(), self._plan.data_ptr(), self._n_items,
-            self._workspace.data_ptr(), self._workspace.numel() * self._workspace.element_size(),
+            self._plan.data_ptr(), self._n_items, self._n_workgroups, self._workspace.data_ptr(), self._workspace.numel() * self._workspace.element_size(),
             self._batch, self._hq, self._hkv, self._d, self._p, scale, _lib.dtype_code(q.dtype),
-            _lib.current_stream())
+            phases, _lib.current_stream())
         _lib.check(rc, "decode forward")
         return out
 

@@ -68,20 +68,23 @@ int dskv_scatter_pages(void *pool, const void *chunk, const int32_t *page_ids, i
  * begin_forward (execution/exec.py:184-192) = dskv_decode_plan, and
  * forward (model/layer/attention.py:185) = dskv_decode_attn.
  *
- * dskv_decode_plan runs on the host from host copies of the CSR metadata and
- * fills plan_host (int32 words) with the split-KV work list; the caller copies
- * it to the device once per step and reuses it for every layer.
- *   plan_capacity_words: size of plan_host; required size is at most
- *                        dskv_decode_plan_bound(batch, total_tokens).
- *   n_items_out:         number of work items (grid size).
- *   workspace_bytes_out: device scratch dskv_decode_attn needs for partials.
- * target_items <= 0 lets the planner choose for the whole chip.
+ * dskv_decode_plan runs on the host from host copies of the CSR metadata.  It
+ * lays all requests' 16-token tiles end to end, cuts the sequence into one equal
+ * share per workgroup and writes the resulting work list to plan_host (int32
+ * words: 4 header words, 8 per item, n_workgroups + 1 share offsets, 2 per
+ * request); the caller copies it to the device once per step and reuses it for
+ * every layer.
+ *   target_workgroups:   <= 0 = one per compute unit of the current device.
+ *   plan_capacity_words: size of plan_host; dskv_decode_plan_bound(batch,
+ *                        total_tokens) words always suffice.
+ *   workspace_bytes_out: device scratch dskv_decode_attn needs for the partial
+ *                        results of requests that were cut.
  */
 int64_t dskv_decode_plan_bound(int32_t batch, int64_t total_tokens);
 int dskv_decode_plan(const int32_t *kv_page_indptr_host, const int32_t *kv_last_page_len_host,
                      int32_t batch, int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
-                     int32_t head_dim, int32_t target_items, int32_t *plan_host,
-                     int64_t plan_capacity_words, int32_t *n_items_out,
+                     int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
+                     int64_t plan_capacity_words, int32_t *n_items_out, int32_t *n_workgroups_out,
                      int64_t *plan_words_out, int64_t *workspace_bytes_out);
 
 /*
@@ -90,11 +93,22 @@ int dskv_decode_plan(const int32_t *kv_page_indptr_host, const int32_t *kv_last_
  * over the kv_len_b tokens fixed at plan time.  fp32 accumulation.
  */
 int dskv_decode_attn(void *out, const void *q, const void *pages_layer,
-                     const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
-                     const int32_t *plan_dev, int32_t n_items, void *workspace,
-                     int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
-                     int32_t n_kv_heads, int32_t head_dim, int32_t page_size, float sm_scale,
-                     int32_t dtype, void *stream);
+                     const int32_t *kv_page_indices, const int32_t *plan_dev, int32_t n_items,
+                     int32_t n_workgroups, void *workspace, int64_t workspace_bytes, int32_t batch,
+                     int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
+                     float sm_scale, int32_t dtype, void *stream);
+/*
+ * The same, one pass at a time: phases bit 0 = the split-KV attention pass
+ * (writes final rows of uncut requests and the partials of cut ones), bit 1 =
+ * the merge pass that combines the partials.  dskv_decode_attn is phases = 3.
+ * Lets a caller time or overlap the two passes separately.
+ */
+int dskv_decode_attn_phases(void *out, const void *q, const void *pages_layer,
+                            const int32_t *kv_page_indices, const int32_t *plan_dev,
+                            int32_t n_items, int32_t n_workgroups, void *workspace,
+                            int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
+                            int32_t n_kv_heads, int32_t head_dim, int32_t page_size, float sm_scale,
+                            int32_t dtype, int32_t phases, void *stream);
 
 /*
  * Paged prefill attention with the end-aligned causal mask.  Replaces

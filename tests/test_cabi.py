@@ -40,12 +40,15 @@ def test_argument_errors_return_negative_codes_without_a_gpu():
     assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 100, 0, 8, None) == -1      # page_bytes % 16
     assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 64, 3, 9, None) == -1       # row range
     assert lib.dskv_scatter_pages(16, 16, 16, 4, 2, 1024, 64, 0, 0, None) == 0       # empty range
-    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 3, None, 0, 2, 32, 8, 128, 16, 0.1, 7, None) == -1
-    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 3, None, 0, 2, 30, 8, 128, 16, 0.1, 2, None) == -1
-    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 5, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
+    # out, q, pages, indices, plan, n_items, n_wgs, ws, ws_bytes, batch, Hq, Hkv, D, P, scale, dtype, stream
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 3, 2, None, 0, 2, 32, 8, 128, 16, 0.1, 7, None) == -1
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 3, 2, None, 0, 2, 30, 8, 128, 16, 0.1, 2, None) == -1
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 5, 2, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
     assert "workspace" in _lib.last_error()
-    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 16, 2, None, 0, 2, 32, 8, 128, 12, 0.1, 2, None) == -1
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 2, 2, None, 0, 2, 32, 8, 128, 12, 0.1, 2, None) == -1
     assert "power-of-two" in _lib.last_error()
+    assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 2, 0, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
+    assert lib.dskv_decode_attn_phases(16, 16, 16, 16, 16, 2, 2, None, 0, 2, 32, 8, 128, 16, 0.1, 2, 0, None) == -1
     assert lib.dskv_apply_rope(16, 16, 16, 16, 16, 16, 1, 1, 32, 8, 130, 5e5, 2, None) == -1
     assert lib.dskv_swap_slice(16, 64, 128, 2, 16, 16, None, None) == -1             # stride < slice
     assert lib.dskv_swap_slice(None, 0, 0, 0, None, None, None, None) == 0
@@ -62,20 +65,25 @@ def _plan(lens, P=16, Hq=32, Hkv=8, D=128, target=0):
     last = np.where(lens > 0, (lens - 1) % P + 1, 0).astype(np.int32)
     cap = lib.dskv_decode_plan_bound(len(lens), int(npages.sum()) * P)
     plan = np.zeros(max(cap, 1), np.int32)
-    n, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+    n, wgs, words, ws = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
     rc = lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, len(lens), P, Hq, Hkv, D, target,
-                              plan.ctypes.data, cap, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+                              plan.ctypes.data, cap, ctypes.byref(n), ctypes.byref(wgs),
+                              ctypes.byref(words), ctypes.byref(ws))
     assert rc == 0, _lib.last_error()
-    items = plan[: n.value * 4].reshape(-1, 4)
-    req = plan[n.value * 4: words.value].reshape(-1, 2)
-    return items, req, ws.value
+    assert plan[:4].tolist()[:2] == [n.value, wgs.value] and plan[3] == len(lens)
+    items = plan[4: 4 + n.value * 8].reshape(-1, 8)
+    wg_ptr = plan[4 + n.value * 8: 4 + n.value * 8 + wgs.value + 1]
+    req = plan[4 + n.value * 8 + wgs.value + 1: words.value].reshape(-1, 2)
+    assert np.array_equal(items[:, 4], indptr[items[:, 0]])          # page_begin = kv_page_indptr[b]
+    return items[:, :4], wg_ptr, req, ws.value, int(plan[2])
 
 
 @pytest.mark.parametrize("lens,target", [([512] * 8, 0), ([1, 15, 16, 17, 4096, 300], 0),
-                                         ([32768, 64, 2048], 64), ([5], 0), ([0, 7], 0),
-                                         (list(range(256, 4097, 61)), 1024)])
-def test_decode_plan_covers_every_token_exactly_once(lens, target):
-    items, req, ws = _plan(lens, target=target)
+                                         ([32768, 64, 2048], 64), ([5], 0), ([0, 7], 0), ([0, 0], 0),
+                                         (list(range(256, 4097, 61)), 256), ([100] * 300, 7),
+                                         ([4096] * 4, 4096)])
+def test_decode_plan_covers_every_token_once_in_equal_shares(lens, target):
+    items, wg_ptr, req, ws, n_slots = _plan(lens, target=target)
     assert req.shape[0] == len(lens)
     covered = {b: [] for b in range(len(lens))}
     slots = []
@@ -94,23 +102,31 @@ def test_decode_plan_covers_every_token_exactly_once(lens, target):
         else:
             assert parts == len(spans)
             assert sorted(s for s, bb in slots if bb == b) == list(range(first, first + parts))
-    assert sorted(s for s, _ in slots) == list(range(len(slots)))              # dense slot numbering
+    assert sorted(s for s, _ in slots) == list(range(len(slots))) and n_slots == len(slots)
     assert ws == len(slots) * 32 * (128 + 2) * 4
-    sizes = [t1 - t0 for _, t0, t1, _ in items]
-    assert sizes == sorted(sizes, reverse=True)                                # longest first
+    # shares: contiguous item ranges, every item owned once, tile counts equal to within one
+    assert wg_ptr[0] == 0 and wg_ptr[-1] == len(items) and np.all(np.diff(wg_ptr) >= 0)
+    tiles = [-(-(t1 - t0) // 16) for _, t0, t1, _ in items]
+    per_wg = [sum(tiles[a:b]) for a, b in zip(wg_ptr[:-1], wg_ptr[1:])]
+    total = sum(tiles)
+    assert sum(per_wg) == total
+    if total:
+        assert max(per_wg) - min(per_wg) <= 1 and min(per_wg) >= min(4, total)
+    assert len(per_wg) <= max(1, total // 4) or len(per_wg) == 1
 
 
 def test_decode_plan_rejects_bad_metadata_and_small_buffers():
     lib = _lib.lib()
     indptr = np.array([0, 2], np.int32)
     last = np.array([17], np.int32)
-    n, words, ws = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+    n, wgs, words, ws = ctypes.c_int32(), ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
     plan = np.zeros(64, np.int32)
-    args = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 64, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+    outs = (ctypes.byref(n), ctypes.byref(wgs), ctypes.byref(words), ctypes.byref(ws))
+    args = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 64) + outs
     assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *args) == -1
     last[0] = 16
     assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *args) == 0
-    small = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 3, ctypes.byref(n), ctypes.byref(words), ctypes.byref(ws))
+    small = (1, 16, 32, 8, 128, 0, plan.ctypes.data, 3) + outs
     assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *small) == -2
 
 
@@ -124,10 +140,16 @@ def test_prefill_plan_tiles_cover_all_query_rows():
         assert lib.dskv_prefill_plan(qo.ctypes.data, 4, hq, hkv, tiles.ctypes.data, cap, ctypes.byref(n)) == 0
         t = tiles[: 2 * n.value].reshape(-1, 2)
         group = hq // hkv
-        rows = 2 * (16 // group) if group <= 16 else 1
+        rows = None
         for b in range(4):
             nb = qo[b + 1] - qo[b]
             starts = sorted(t[t[:, 0] == b][:, 1].tolist())
+            if nb == 0:
+                assert starts == []
+                continue
+            if rows is None:
+                rows = starts[1] - starts[0] if len(starts) > 1 else nb
+                assert rows % max(16 // group, 1) == 0 if group <= 16 else rows == 1
             assert starts == list(range(0, nb, rows))
     n = ctypes.c_int32()
     assert lib.dskv_prefill_plan(qo.ctypes.data, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2

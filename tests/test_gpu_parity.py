@@ -97,14 +97,14 @@ def test_gather_scatter_bit_exact(dtype, P):
 
 
 # ------------------------------------------------------------------ decode attention
-def _run_decode(sc, target_items=0):
+def _run_decode(sc, target_items=0):   # target_items = persistent workgroups (0: one per CU)
     from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
 
     ws = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
     w = BatchDecodeWithPagedKVCacheWrapper(ws)
     w.begin_forward(_dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                     _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P,
-                    target_items=target_items)
+                    target_workgroups=target_items)
     out = w.forward(to_torch(sc.q, sc.dtype), to_torch(sc.pages, sc.dtype))
     w.end_forward()
     torch.cuda.synchronize()
@@ -145,7 +145,7 @@ def test_decode_attention_matches_oracle(case):
     assert not got[~live].any()                       # a request without tokens yields zeros
     if name == "split":
         assert n_items > len(lens)
-    if name == "nosplit":
+    if name == "nosplit":                  # a single workgroup: no request is cut
         assert n_items == len(lens)
 
 
@@ -194,7 +194,7 @@ def test_decode_wrapper_protocol_errors():
     small = BatchDecodeWithPagedKVCacheWrapper(torch.empty(1024, dtype=torch.uint8, device="cuda"))
     with pytest.raises(RuntimeError, match="workspace"):
         small.begin_forward(_dev_i32([0, 256]), _dev_i32(list(range(256))), _dev_i32([16]), 32, 8,
-                            128, 16, target_items=8)
+                            128, 16, target_workgroups=8)
     with pytest.raises(ValueError):
         w.begin_forward(_dev_i32([0, 1]), _dev_i32([2]), _dev_i32([17]), 32, 8, 128, 16)
 
@@ -237,7 +237,7 @@ def test_prefill_with_one_query_equals_decode():
 
     _announce("prefill n=1 vs decode")
     sc = make_scenario(42, kv_lens=[700, 33, 16], qo_lens=[1, 1, 1], dtype="bf16")
-    dec, _ = _run_decode(sc, target_items=1)
+    dec, _ = _run_decode(sc, 1)
     w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
     w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                     _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P)
