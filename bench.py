@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
     ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="before the timed region run one plain page-copy kernel of known size "
+                         "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="do not bracket the attention pass with events (pure step timing)")
     return ap.parse_args()
@@ -122,6 +125,16 @@ def main() -> int:
     e = wl.pool.pages.element_size()
     tok_bytes = wl.kv_bytes_per_token()
     torch.cuda.synchronize()
+
+    if a.pmc_calibration:
+        # move_pages_kernel<true> over 4096 consecutive 64 KiB pages of layer 0 -> scratch
+        from deserve_amd.kvcache import _native
+        ids = torch.arange(4096, dtype=torch.int32)
+        one_layer = type("OneLayer", (), {"num_layers": 1, "pages": wl.pool.pages[:1],
+                                          "layer_stride_bytes": wl.pool.layer_stride_bytes,
+                                          "page_bytes": wl.pool.page_bytes})()
+        _native.gather_pages(one_layer, ids)
+        torch.cuda.synchronize()
 
     ev_pairs = []          # (start, end) events around the split-KV attention pass
     step_bytes = []
