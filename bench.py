@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
     ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -98,6 +99,114 @@ def cpu_baseline(wl, meta, sample_requests: int):
                       f"{med * 1e3:.1f} ms each, scalar C + OpenMP"}
 
 
+def swap_section(seed: int):
+    """Baseline configuration 3 (Llama-3-70B stage, 10 layers, GQA 64q/8kv): one microbatch's
+    scattered pages go out to pinned host memory while the next one's come in (one
+    exchange call), overlapped with decode steps of the resident microbatch."""
+    import numpy as np
+    import torch
+
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.kvcache import _native
+    from deserve_amd.kvcache.pinned.pinned_memory import pinned_empty
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.paged_ops import append_paged_kv_cache
+    from deserve_amd.synthetic import make_decode_workload
+
+    L, Hq, Hkv, D, P = 10, 64, 8, 128, 16
+    rng = np.random.default_rng(seed + 30)
+    ctx = rng.integers(1024, 4097, size=32)                 # resident microbatch
+    other = rng.integers(1024, 4097, size=32)               # the microbatch being exchanged
+    n_swap = int((-(-other // P)).sum())
+    wl = make_decode_workload("cfg3", ctx, L, Hq, Hkv, D, P, torch.bfloat16, headroom_tokens=512,
+                              seed=seed, spare_pages=n_swap + 64, fill=False)
+    wl.pool.pages.zero_()
+    ids = wl.pool.alloc(n_swap)                             # scattered: the pool hands out a permutation
+    shape = (L * n_swap,) + tuple(wl.pool.pages.shape[2:])
+    host_out, host_in = pinned_empty(shape, torch.bfloat16), pinned_empty(shape, torch.bfloat16)
+    host_in.zero_()
+    nbytes = host_out.numel() * 2
+    eng = _native.SwapEngine()
+    w, _ = get_wrappers(wl.pool.main_device)
+
+    def decode_step():
+        c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, w)
+        w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
+                        last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
+                        head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
+                        last_page_len_host=c.host["kv_last_page_lens"])
+        for layer in range(L):
+            pages = wl.pool.get_layered_pages(layer)
+            append_paged_kv_cache(wl.k[layer], wl.v[layer], c.indptr, pages, c.kv_page_indices,
+                                  c.kv_page_indptr, c.kv_last_page_lens)
+            w.forward(wl.q[layer], pages)
+        w.end_forward()
+        for t in wl.tasks:
+            t.step()
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    # host-link denominator: plain pinned copies of the same size, both directions at once
+    dev_a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dev_b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    flat_out, flat_in = host_out.view(torch.uint8).view(-1), host_in.view(torch.uint8).view(-1)
+
+    def raw_duplex():
+        with torch.cuda.stream(s1):
+            flat_out.copy_(dev_a, non_blocking=True)
+        with torch.cuda.stream(s2):
+            dev_b.copy_(flat_in, non_blocking=True)
+
+    raw_duplex()
+    link = nbytes / min(timed(raw_duplex) for _ in range(2)) / 1e9
+    del dev_a, dev_b
+
+    def exchange():
+        eng.exchange(host_out, host_in, wl.pool, ids)
+        eng.wait()
+
+    exchange()
+    alone = nbytes / min(timed(exchange) for _ in range(2)) / 1e9
+    for _ in range(3):
+        decode_step()
+    t_dec = timed(lambda: [decode_step() for _ in range(10)]) / 10
+
+    # overlapped: start the exchange, decode until it has finished
+    torch.cuda.synchronize()
+    done = torch.cuda.Event()
+    t0 = time.perf_counter()
+    eng.exchange(host_out, host_in, wl.pool, ids)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        eng.fence()                 # the side stream (not the compute stream) waits for the swap
+        done.record()
+    steps = 0
+    while not done.query():
+        decode_step()
+        steps += 1
+    done.synchronize()
+    t_swap = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    t_all = time.perf_counter() - t0
+    eng.close()
+    return {"workload": "BASELINE.json configs[2]: 10 layers, bf16, GQA 64q/8kv, page 16, microbatch of 32 "
+                        "sequences ctx U[1024,4096]; scattered pages out + next microbatch in, one exchange",
+            "pages": n_swap, "bytes_each_way": nbytes,
+            "host_link_duplex_GBps_each_way": round(link, 2),
+            "exchange_alone_GBps_each_way": round(alone, 2),
+            "exchange_overlapped_GBps_each_way": round(nbytes / t_swap / 1e9, 2),
+            "frac_of_host_link_overlapped": round(nbytes / t_swap / 1e9 / link, 3),
+            "decode_ms_per_step_alone": round(t_dec * 1e3, 3),
+            "decode_ms_per_step_during_swap": round(t_all / max(steps, 1) * 1e3, 3),
+            "decode_steps_during_swap": steps}
+
+
 def main() -> int:
     a = parse_args()
     if a.gpus != 1:
@@ -136,7 +245,11 @@ def main() -> int:
         _native.gather_pages(one_layer, ids)
         torch.cuda.synchronize()
 
-    ev_pairs = []          # (start, end) events around the split-KV attention pass
+    # (start, end) events around the split-KV attention pass, created before the timed region
+    ev_pool = [] if a.no_kernel_events else [
+        (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+        for _ in range(a.steps * L)]
+    ev_pairs = []
     step_bytes = []
     attn_bytes_layer = []
 
@@ -157,7 +270,7 @@ def main() -> int:
             append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
                                   c.kv_last_page_lens)
             if timed and not a.no_kernel_events:
-                s, t = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s, t = ev_pool[len(ev_pairs)]
                 s.record()
                 out = decode_wrapper.forward(q, pages, phases=1)
                 t.record()
@@ -218,6 +331,10 @@ def main() -> int:
     if not a.no_cpu_baseline:
         meta = {n: last_ctx.host[n].numpy() for n in ("kv_page_indices", "kv_page_indptr", "kv_last_page_lens")}
         out["cpu_baseline"] = cpu_baseline(wl, meta, sample_requests=16)
+    if not a.no_swap:
+        del wl, last_ctx
+        torch.cuda.empty_cache()
+        out["swap"] = swap_section(a.seed)
     print(json.dumps(out))
     return 0
 

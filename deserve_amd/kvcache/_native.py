@@ -50,7 +50,7 @@ def scatter_pages(pool, ids: torch.Tensor, chunk: torch.Tensor) -> None:
 class SwapEngine:
     """Owner of one dskv_swap handle (side streams + staging buffers)."""
 
-    def __init__(self, staging_bytes: int = 64 << 20) -> None:
+    def __init__(self, staging_bytes: int = 128 << 20) -> None:
         import ctypes
 
         h = ctypes.c_void_p()

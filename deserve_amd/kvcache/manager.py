@@ -23,7 +23,7 @@ from deserve_amd.kvcache.virtual import VirtualPagedKVCache, VirtualPagePool
 
 class KVCacheManager:
     def __init__(self, virtual_page_pool: VirtualPagePool, cpu_chunk_pool: CpuChunkPool,
-                 page_table_allocator: PageTableAllocator, staging_bytes: int = 64 << 20):
+                 page_table_allocator: PageTableAllocator, staging_bytes: int = 128 << 20):
         self.virtual_page_pool = virtual_page_pool
         self.cpu_chunk_pool = cpu_chunk_pool
         self.page_table_allocator = page_table_allocator
