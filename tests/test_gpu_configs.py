@@ -1,0 +1,302 @@
+"""The baseline configurations at their FULL sizes on one MI355X.  The CPU oracle
+cannot redo gigabytes in seconds, so parity is shown through (a) the oracle on a
+seeded sample of requests / query rows, (b) size-independent properties:
+append -> read-back identity plus a checksum of everything that must not change,
+swap round trips that must restore every bit, and invariance of attention under
+relocation of the pages."""
+import numpy as np
+import pytest
+import torch
+
+from kvutil import from_torch, max_rel_err
+from oracle import c_oracle
+from oracle import kv_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda")
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def _checksum(t: torch.Tensor) -> int:
+    """Order-independent 64-bit sum of the raw 16-bit words."""
+    return int(t.contiguous().view(torch.int16).to(torch.int64).sum().item())
+
+
+def _bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _decode_step(wl, wrapper, layers, rope=False):
+    """One engine-style decode step over the given layers; returns (ctx, {layer: out})."""
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.paged_ops import append_paged_kv_cache
+
+    a = wl.args
+    ctx = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, wrapper)
+    wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ctx.kv_page_indices,
+                          last_page_len=ctx.kv_last_page_lens, num_qo_heads=a.n_heads,
+                          num_kv_heads=a.n_kv_heads, head_dim=a.dim // a.n_heads, page_size=a.page_size,
+                          indptr_host=ctx.host["kv_page_indptr"],
+                          last_page_len_host=ctx.host["kv_last_page_lens"])
+    outs = {}
+    for layer in layers:
+        pages = wl.pool.get_layered_pages(layer)
+        append_paged_kv_cache(wl.k[layer], wl.v[layer], ctx.indptr, pages, ctx.kv_page_indices,
+                              ctx.kv_page_indptr, ctx.kv_last_page_lens)
+        outs[layer] = wrapper.forward(wl.q[layer], pages)
+    wrapper.end_forward()
+    torch.cuda.synchronize()
+    return ctx, outs
+
+
+def _oracle_rows(wl, ctx, layer, requests):
+    """fp32 oracle output for a sample of requests: their pages are copied to the host."""
+    P = wl.args.page_size
+    indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
+    last = ctx.host["kv_last_page_lens"].numpy()
+    want = {}
+    for b in requests:
+        ids = ids_all[indptr[b]: indptr[b + 1]]
+        pages = _bits(wl.pool.pages[layer].index_select(0, torch.from_numpy(ids.astype(np.int64)).to(DEV)))
+        q = _bits(wl.q[layer, b: b + 1])
+        want[b] = c_oracle.decode_attn(q, pages, np.arange(len(ids), dtype=np.int32),
+                                       np.array([0, len(ids)], np.int32), last[b: b + 1], "bf16")[0]
+    return want
+
+
+def _check_append(wl, ctx, layer, before_sum, old_rows):
+    """The new rows read back through the block table equal k/v bit for bit, and the
+    checksum of the whole layer moved by exactly (new rows - old rows)."""
+    P = wl.args.page_size
+    indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
+    last = ctx.host["kv_last_page_lens"].numpy()
+    page = torch.from_numpy(ids_all[indptr[1:] - 1].astype(np.int64)).to(DEV)
+    slot = torch.from_numpy((last - 1).astype(np.int64)).to(DEV)
+    got = wl.pool.pages[layer][page, :, slot]                       # (B, 2, Hkv, D)
+    assert torch.equal(got[:, 0].view(torch.int16), wl.k[layer].view(torch.int16))
+    assert torch.equal(got[:, 1].view(torch.int16), wl.v[layer].view(torch.int16))
+    delta = _checksum(wl.k[layer]) + _checksum(wl.v[layer]) - old_rows
+    assert _checksum(wl.pool.pages[layer]) == before_sum + delta, "bytes outside the new rows changed"
+
+
+def _old_rows_sum(wl, layer):
+    """Checksum of the slots the next append will overwrite (position start_pos of every request)."""
+    P = wl.args.page_size
+    total = 0
+    pages, slots = [], []
+    for t, c in zip(wl.tasks, wl.caches):
+        c.extend(t.start_pos + 1)                     # what prepare() will do
+        pages.append(int(c.page_table.retrieve()[t.start_pos // P]))
+        slots.append(t.start_pos % P)
+    rows = wl.pool.pages[layer][torch.tensor(pages, device=DEV), :, torch.tensor(slots, device=DEV)]
+    return _checksum(rows)
+
+
+def test_config2_llama8b_stage_decode_step_full_size():
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.synthetic import config2_context_lengths, make_decode_workload
+
+    _announce("config2 full size")
+    wl = make_decode_workload("cfg2", config2_context_lengths(2), 16, 32, 8, 128, 16, torch.bfloat16,
+                              headroom_tokens=32, seed=2)
+    wrapper, _ = get_wrappers(DEV)
+    layers = [0, 7, 15]
+    before = {l: _checksum(wl.pool.pages[l]) for l in layers}
+    old = {l: _old_rows_sum(wl, l) for l in layers}
+    ctx, outs = _decode_step(wl, wrapper, layers)
+    sample = [int(np.argmax(wl.ctx_lens)), int(np.argmin(wl.ctx_lens)), 5]
+    for l in layers:
+        _check_append(wl, ctx, l, before[l], old[l])
+    want = _oracle_rows(wl, ctx, 7, sample)
+    got = outs[7].float().cpu().numpy()
+    for b in sample:
+        assert max_rel_err(got[b], want[b]) <= 2e-2, b
+    assert torch.isfinite(outs[0].float()).all() and torch.isfinite(outs[15].float()).all()
+    # relocating every page of the layer (and renaming it in the block table) changes nothing
+    perm = torch.randperm(wl.pool.num_pages, device=DEV)
+    moved = torch.empty_like(wl.pool.pages[7])
+    moved[perm] = wl.pool.pages[7]
+    new_ids = perm[ctx.kv_page_indices.long()].to(torch.int32)
+    wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=new_ids, last_page_len=ctx.kv_last_page_lens,
+                          num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
+                          indptr_host=ctx.host["kv_page_indptr"], last_page_len_host=ctx.host["kv_last_page_lens"])
+    again = wrapper.forward(wl.q[7], moved)
+    wrapper.end_forward()
+    assert torch.equal(again.view(torch.int16), outs[7].view(torch.int16))
+
+
+def test_config3_microbatch_exchange_round_trip_full_size():
+    """4648+ scattered pages x 10 layers (~3 GB) out and back in: every bit restored,
+    while the pages of the resident microbatch are never touched."""
+    from deserve_amd.kvcache import _native
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.pinned.pinned_memory import pinned_empty
+    from deserve_amd.synthetic import fill_normal, scatter_pool_order
+
+    _announce("config3 full size")
+    L, P = 10, 16
+    rng = np.random.default_rng(3)
+    n_mb = [int((-(-rng.integers(1024, 4097, size=32) // P)).sum()) for _ in range(2)]
+    pool = GpuPagePool(L, sum(n_mb) + 100, P, DEV, torch.bfloat16)
+    fill_normal(pool.pages, 3)
+    scatter_pool_order(pool, 4)
+    ids_a, ids_b = pool.alloc(n_mb[0]), pool.alloc(n_mb[1])
+    sum_all = _checksum(pool.pages)
+    image_a = pool.retrieve(ids_a)                                  # device copy (L, n, ...)
+    sum_b = _checksum(pool.retrieve(ids_b))
+    eng = _native.SwapEngine()
+    shape = (L * n_mb[0],) + tuple(pool.pages.shape[2:])
+    host_a, host_z = pinned_empty(shape, torch.bfloat16), pinned_empty(shape, torch.bfloat16)
+    host_z.zero_()
+    eng.exchange(host_a, host_z, pool, ids_a)                       # a goes out, zeros come in
+    eng.wait()
+    assert _checksum(pool.retrieve(ids_a)) == 0
+    assert _checksum(pool.retrieve(ids_b)) == sum_b                 # resident microbatch untouched
+    assert torch.equal(host_a.view(torch.int16).view(image_a.shape), image_a.cpu().view(torch.int16))
+    eng.exchange(host_z, host_a, pool, ids_a)                       # and back
+    eng.wait()
+    assert torch.equal(pool.retrieve(ids_a).view(torch.int16), image_a.view(torch.int16))
+    assert _checksum(pool.pages) == sum_all
+    eng.close()
+
+
+def test_config4_chunked_prefill_full_batch_two_layers():
+    """16 sequences append a 512-token chunk behind a prior of U[0, 8192] tokens that ends
+    mid-page (offset U[0, 15]), then attend causally over prior + chunk."""
+    from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.model.context.flash import FlashPrefillCtx
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper, append_paged_kv_cache
+    from deserve_amd.synthetic import fill_normal, scatter_pool_order
+    from deserve_amd.task import SamplingParams, TaskData
+
+    _announce("config4")
+    L, P, Hq, Hkv, D, B, n = 2, 16, 32, 8, 128, 16, 512
+    rng = np.random.default_rng(4)
+    prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
+    prior[0], prior[1] = 0, 8192 + 15                               # extremes: pure prompt, longest
+    pool = GpuPagePool(L, int((-(-(prior + n) // P)).sum()) + 8, P, DEV, torch.bfloat16)
+    fill_normal(pool.pages, 5)
+    scatter_pool_order(pool, 6)
+    rows = PageTableAllocator(B, 8192 + 1024, P, DEV)
+    tasks = [TaskData(f"t{b}", int(prior[b]), 1, n, int(prior[b]) + n, SamplingParams()) for b in range(B)]
+    caches = [PagedKVCache.empty(rows, pool) for _ in range(B)]
+    g = torch.Generator(device=DEV)
+    g.manual_seed(7)
+    mk = lambda h: torch.randn((L, B * n, h, D), generator=g, device=DEV).to(torch.bfloat16)
+    q, k, v = mk(Hq), mk(Hkv), mk(Hkv)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device=DEV))
+    ctx = FlashPrefillCtx.init_paged_prefill_ctx(tasks, caches, w)
+    w.begin_forward(qo_indptr=ctx.indptr, paged_kv_indptr=ctx.kv_page_indptr,
+                    paged_kv_indices=ctx.kv_page_indices, paged_kv_last_page_len=ctx.kv_last_page_lens,
+                    num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
+                    qo_indptr_host=ctx.host["indptr"])
+    before = [_checksum(pool.pages[l]) for l in range(L)]
+    indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
+    # slots the chunk will overwrite: positions prior_b .. prior_b + n - 1
+    pos = np.concatenate([np.arange(p, p + n) for p in prior])
+    req = np.repeat(np.arange(B), n)
+    page = torch.from_numpy(ids_all[indptr[req] + pos // P].astype(np.int64)).to(DEV)
+    slot = torch.from_numpy((pos % P).astype(np.int64)).to(DEV)
+    outs = []
+    for l in range(L):
+        old = _checksum(pool.pages[l][page, :, slot])
+        append_paged_kv_cache(k[l], v[l], ctx.indptr, pool.pages[l], ctx.kv_page_indices,
+                              ctx.kv_page_indptr, ctx.kv_last_page_lens)
+        got = pool.pages[l][page, :, slot]
+        assert torch.equal(got[:, 0].view(torch.int16), k[l].view(torch.int16))
+        assert torch.equal(got[:, 1].view(torch.int16), v[l].view(torch.int16))
+        assert _checksum(pool.pages[l]) == before[l] - old + _checksum(k[l]) + _checksum(v[l])
+        outs.append(w.forward(q[l], pool.pages[l], causal=True))
+    torch.cuda.synchronize()
+    w.end_forward()
+    # oracle on sampled query rows: row i of request b is decode attention over prior_b + i + 1 tokens
+    layer = 1
+    got = outs[layer].float().cpu().numpy()
+    for b, i in [(0, 0), (0, 511), (1, 0), (1, 300), (1, 511), (7, 17), (15, 256)]:
+        limit = int(prior[b]) + i + 1
+        npg = -(-limit // P)
+        ids = ids_all[indptr[b]: indptr[b] + npg]
+        pages = _bits(pool.pages[layer].index_select(0, torch.from_numpy(ids.astype(np.int64)).to(DEV)))
+        row = b * n + i
+        want = c_oracle.decode_attn(_bits(q[layer, row: row + 1]), pages, np.arange(npg, dtype=np.int32),
+                                    np.array([0, npg], np.int32),
+                                    np.array([(limit - 1) % P + 1], np.int32), "bf16")[0]
+        assert max_rel_err(got[row], want) <= 2e-2, (b, i)
+    assert np.isfinite(got).all()
+
+
+def test_config5_fragmented_pool_swap_in_then_decode():
+    """128 sequences with lognormal context lengths on a pool fragmented by evictions
+    (40 % of the pages freed and re-allocated out of order); 25 % of the sequences are
+    offloaded and reloaded into other pages before the decode step."""
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.kvcache.manager import KVCacheManager
+    from deserve_amd.kvcache.paged.chunk_pool import CpuChunkPool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.kvcache.virtual import VirtualPagedKVCache, VirtualPagePool
+    from deserve_amd.stage import KVStage, StageArgs
+    from deserve_amd.synthetic import DecodeWorkload, config5_context_lengths, fill_normal
+    from deserve_amd.task import SamplingParams, TaskData
+
+    _announce("config5")
+    L, P, Hq, Hkv, D, B = 10, 16, 64, 8, 128, 128
+    rng = np.random.default_rng(5)
+    ctx_lens = config5_context_lengths(5)
+    need = int((-(-(ctx_lens + 8) // P)).sum())
+    pool = VirtualPagePool(L, int(need / 0.4 * 1.05) + 128, 0, P, DEV, torch.bfloat16)   # 40 % of it must hold everything
+    fill_normal(pool.pages, 8)
+    rows = PageTableAllocator(B + 40, 32768 + 64, P, DEV)
+    # fragmentation: fill the pool with filler requests, free a seeded 40 % of all pages,
+    # then allocate the real requests (they get the lowest free ids first = holes all over)
+    filler = pool.alloc(pool.num_avails)
+    freed = torch.from_numpy(rng.permutation(filler.numpy())[: int(0.4 * len(filler))].copy())
+    pool.free(freed)
+    tasks, caches = [], []
+    order = rng.permutation(B)                         # out-of-order arrival
+    made = {}
+    for b in order:
+        c = VirtualPagedKVCache.empty(rows, pool)
+        c.extend(int(ctx_lens[b]))
+        made[int(b)] = c
+    for b in range(B):
+        tasks.append(TaskData(f"t{b}", int(ctx_lens[b]), 1, 1, int(ctx_lens[b]), SamplingParams()))
+        caches.append(made[b])
+    ids0 = caches[0].page_table.retrieve().numpy()
+    assert np.any(np.diff(ids0) != 1), "block table should be fragmented"
+    mgr = KVCacheManager(pool, CpuChunkPool(L, 14, P, torch.bfloat16), rows)
+    swapped = sorted(rng.choice(B, size=B // 4, replace=False).tolist())
+    images = {b: pool.retrieve(caches[b].page_table.retrieve()) for b in swapped[:4]}
+    handles = [mgr.copy_gpu_to_cpu(caches[b], tasks[b].task_id) for b in swapped]
+    for b in swapped:
+        caches[b].free()
+    back = [mgr.copy_cpu_to_gpu(h, tasks[b].task_id) for h, b in zip(handles, swapped)]
+    for h in handles:
+        h.free()
+    mgr.synchronize()
+    for b, c in zip(swapped, back):
+        caches[b] = c
+    for b in swapped[:4]:
+        assert torch.equal(pool.retrieve(caches[b].page_table.retrieve()).view(torch.int16),
+                           images[b].view(torch.int16)), "swap-in changed the data"
+    g = torch.Generator(device=DEV)
+    g.manual_seed(9)
+    mk = lambda h: torch.randn((L, B, h, D), generator=g, device=DEV).to(torch.bfloat16)
+    args = StageArgs(n_heads=Hq, n_kv_heads=Hkv, dim=Hq * D, page_size=P, n_layers=L)
+    wl = DecodeWorkload("cfg5", args, pool, rows, tasks, caches, KVStage(args, use_rope=False),
+                        mk(Hq), mk(Hkv), mk(Hkv), ctx_lens)
+    wrapper, _ = get_wrappers(DEV)
+    layer = 4
+    before, old = _checksum(pool.pages[layer]), _old_rows_sum(wl, layer)
+    ctx, outs = _decode_step(wl, wrapper, [layer])
+    _check_append(wl, ctx, layer, before, old)
+    sample = [int(np.argmax(ctx_lens)), int(np.argmin(ctx_lens)), swapped[0], swapped[-1]]
+    want = _oracle_rows(wl, ctx, layer, sample)
+    got = outs[layer].float().cpu().numpy()
+    for b in sample:
+        assert max_rel_err(got[b], want[b]) <= 2e-2, b
+    assert np.isfinite(got).all()
