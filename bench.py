@@ -33,8 +33,8 @@ HBM_PEAK_GBPS = 8000.0
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
     ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
@@ -45,6 +45,10 @@ def parse_args():
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
     ap.add_argument("--no-kernel-events", action="store_true",
                     help="do not bracket the attention pass with events (pure step timing)")
+    ap.add_argument("--event-every", type=int, default=4,
+                    help="bracket every Nth attention launch with events; the host must stay ahead "
+                         "of the GPU for the event interval to be the kernel alone, so not every "
+                         "launch is bracketed")
     return ap.parse_args()
 
 
@@ -248,8 +252,9 @@ def main() -> int:
     # (start, end) events around the split-KV attention pass, created before the timed region
     ev_pool = [] if a.no_kernel_events else [
         (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-        for _ in range(a.steps * L)]
+        for _ in range(a.steps * L // max(a.event_every, 1) + 1)]
     ev_pairs = []
+    launch_no = [0]
     step_bytes = []
     attn_bytes_layer = []
 
@@ -269,7 +274,8 @@ def main() -> int:
             pages = wl.pool.get_layered_pages(layer)
             append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
                                   c.kv_last_page_lens)
-            if timed and not a.no_kernel_events:
+            launch_no[0] += 1
+            if timed and not a.no_kernel_events and launch_no[0] % max(a.event_every, 1) == 0:
                 s, t = ev_pool[len(ev_pairs)]
                 s.record()
                 out = decode_wrapper.forward(q, pages, phases=1)

@@ -41,7 +41,10 @@
 namespace dskv {
 
 constexpr int kMaxWaves = 8;         // kv heads per workgroup
-constexpr int kStages = 3;           // tiles in flight per wave (one consumed, two loading)
+#ifndef DSKV_DECODE_STAGES
+#define DSKV_DECODE_STAGES 3
+#endif
+constexpr int kStages = DSKV_DECODE_STAGES;   // tiles in flight per wave (one consumed, the rest loading)
 constexpr int kPlanHeaderWords = 4;  // n_items, n_workgroups, n_slots, batch
 constexpr int kItemWords = 8;
 constexpr int kMaxWorkgroups = 4096;

