@@ -1,0 +1,142 @@
+"""The stage driver in the reference's call order (synchronize/switch -> adjust ->
+cancel/offload/reload -> join -> prepare -> swap2 -> forward) over rotating
+microbatches: every microbatch must see exactly its own KV, whichever swap slice
+it currently lives in.  Expected outputs come from a shadow copy of each
+request's K/V rows kept in numpy, independent of any page layout."""
+import numpy as np
+import pytest
+import torch
+
+from kvutil import max_rel_err
+from oracle import kv_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda")
+L, P, HQ, HKV, D = 2, 16, 32, 8, 128
+
+
+def _bf(x):
+    return orc.bf16_bits_from_f32(x)
+
+
+def _to_dev(bits):
+    return torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).to(DEV)
+
+
+class Shadow:
+    """Per request and layer: all K/V rows appended so far (bf16 bit patterns)."""
+
+    def __init__(self):
+        self.k = {}
+        self.v = {}
+
+    def expect(self, tid, layer, q_bits, k_bits, v_bits):
+        key = (tid, layer)
+        self.k[key] = np.concatenate([self.k.get(key, np.zeros((0, HKV, D), np.uint16)), k_bits])
+        self.v[key] = np.concatenate([self.v.get(key, np.zeros((0, HKV, D), np.uint16)), v_bits])
+        T, n = self.k[key].shape[0], q_bits.shape[0]
+        npg = -(-T // P)
+        kk = np.zeros((npg * P, HKV, D), np.uint16)
+        vv = np.zeros((npg * P, HKV, D), np.uint16)
+        kk[:T], vv[:T] = self.k[key], self.v[key]
+        pages = np.stack([kk.reshape(npg, P, HKV, D), vv.reshape(npg, P, HKV, D)], axis=1)
+        return orc.prefill_attention(q_bits, np.array([0, n], np.int32), pages,
+                                     np.arange(npg, dtype=np.int32), np.array([0, npg], np.int32),
+                                     np.array([(T - 1) % P + 1], np.int32), "bf16", causal=True)
+
+
+@pytest.mark.parametrize("rounds", [2, 3, 4])
+def test_rotating_microbatches_keep_their_kv(rounds):
+    from deserve_amd.engine.pipeline.processor import PipelineProcessor, StepRequest
+    from deserve_amd.stage import KVStage, StageArgs
+    from deserve_amd.task import SamplingParams
+
+    print("[case] engine rounds", rounds, flush=True)
+    rng = np.random.default_rng(100 + rounds)
+    stage = KVStage(StageArgs(n_heads=HQ, n_kv_heads=HKV, dim=HQ * D, page_size=P, n_layers=L),
+                    use_rope=False)
+    # a tiny main region forces every microbatch into the swap slices
+    proc = PipelineProcessor(num_rounds=rounds, num_pages_main=3, num_pages_swap=24, page_size=P,
+                             batch_size=2, layer_storage=stage, num_layers=L, buddy_height=6,
+                             main_dtype=torch.bfloat16, max_context_len=512)
+    proc.virtual_page_pool.pages.view(torch.int16).fill_(0x7FC0)      # NaN everywhere: stale reads show
+    shadow = Shadow()
+    prompts = {m: {f"m{m}r{r}": int(rng.integers(20, 90)) for r in range(2)} for m in range(rounds)}
+    used_swap_pages = False
+    for step in range(rounds * 6):
+        m = step % rounds
+        first = step < rounds
+        ids = list(prompts[m].keys())
+        seqlens = [prompts[m][t] if first else 1 for t in ids]
+        nnz = sum(seqlens)
+        q = _bf(rng.standard_normal((L, nnz, HQ, D)).astype(np.float32))
+        k = _bf(rng.standard_normal((L, nnz, HKV, D)).astype(np.float32))
+        v = _bf(rng.standard_normal((L, nnz, HKV, D)).astype(np.float32))
+        req = StepRequest(microbatch_id=m, xs=(_to_dev(q), _to_dev(k), _to_dev(v)), exec_task_ids=ids,
+                          exec_seqlens=seqlens,
+                          init_tasks={t: (prompts[m][t], SamplingParams()) for t in ids} if first else {})
+        proc.run_step(req)
+        torch.cuda.synchronize()
+        got = proc.last_result.all_xs.float().cpu().numpy().reshape(L, nnz, HQ, D)
+        assert np.isfinite(got).all(), (step, "a stale or foreign page was read")
+        pos = 0
+        for t, n in zip(ids, seqlens):
+            for layer in range(L):
+                want = shadow.expect(t, layer, q[layer, pos: pos + n], k[layer, pos: pos + n],
+                                     v[layer, pos: pos + n])
+                assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
+            pos += n
+        for c in proc.microbatches[m].ongoing_paged_kvcaches.values():
+            used_swap_pages |= bool(c.isswap[: c.page_table.occupied].any())
+    assert used_swap_pages, "the scenario was meant to exercise the swap slices"
+    proc.synchronize()
+
+
+def test_offload_reload_and_cancel_through_the_stage_driver():
+    from deserve_amd.engine.pipeline.processor import PipelineProcessor, StepRequest
+    from deserve_amd.stage import KVStage, StageArgs
+    from deserve_amd.task import SamplingParams
+
+    print("[case] engine offload/reload", flush=True)
+    rng = np.random.default_rng(7)
+    stage = KVStage(StageArgs(n_heads=HQ, n_kv_heads=HKV, dim=HQ * D, page_size=P, n_layers=L),
+                    use_rope=False)
+    proc = PipelineProcessor(num_rounds=2, num_pages_main=40, num_pages_swap=8, page_size=P,
+                             batch_size=4, layer_storage=stage, num_layers=L, buddy_height=6,
+                             main_dtype=torch.bfloat16, max_context_len=512)
+    shadow = Shadow()
+    lens = {"a": 50, "b": 33, "c": 70}
+
+    def run(m, ids, seqlens, init=False, **kw):
+        nnz = sum(seqlens)
+        q = _bf(rng.standard_normal((L, nnz, HQ, D)).astype(np.float32))
+        k = _bf(rng.standard_normal((L, nnz, HKV, D)).astype(np.float32))
+        v = _bf(rng.standard_normal((L, nnz, HKV, D)).astype(np.float32))
+        req = StepRequest(m, (_to_dev(q), _to_dev(k), _to_dev(v)), ids, seqlens,
+                          init_tasks={t: (lens[t], SamplingParams()) for t in ids} if init else {}, **kw)
+        proc.run_step(req)
+        torch.cuda.synchronize()
+        got = proc.last_result.all_xs.float().cpu().numpy().reshape(L, nnz, HQ, D)
+        pos = 0
+        for t, n in zip(ids, seqlens):
+            for layer in range(L):
+                want = shadow.expect(t, layer, q[layer, pos: pos + n], k[layer, pos: pos + n],
+                                     v[layer, pos: pos + n])
+                assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (t, layer)
+            pos += n
+
+    idle = lambda m, **kw: proc.run_step(StepRequest(m, None, **kw))
+    run(0, ["a", "b", "c"], [50, 33, 70], init=True)
+    idle(1)
+    avail = proc.virtual_page_pool.num_avails
+    run(0, ["a", "c"], [1, 1], offload_task_ids=["b"])              # b leaves for pinned memory
+    assert "b" in proc.offloaded_kvcaches and proc.virtual_page_pool.num_avails >= avail + 3 - 2
+    idle(1)
+    run(0, ["a", "c"], [1, 1])
+    idle(1)
+    run(0, ["a", "b", "c"], [1, 1, 1], reload_task_ids=["b"])       # b comes back into other pages
+    assert not proc.offloaded_kvcaches
+    idle(1)
+    run(0, ["a", "b"], [1, 1], cancel_task_ids=["c"])
+    assert "c" not in proc.microbatches[0].ongoing_paged_kvcaches
+    assert proc.cpu_chunk_pool.available_ids[-1] == [0]              # the chunk was returned
