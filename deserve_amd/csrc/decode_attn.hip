@@ -329,10 +329,10 @@ __global__ __launch_bounds__(64) void decode_attn_generic_kernel(
     }
 }
 
-// Combine the partials of split requests.  One wavefront per (request, q head):
-// lane s first fetches (m, l) of part s, so the maximum and the weights come
-// from one round of independent loads; the O rows are then accumulated with the
-// loads of several parts in flight.
+// Combine the partials of split requests.  One wavefront per (request, q head),
+// lane = 2 dims.  Latency-bound, so dependent memory round trips are kept to
+// two: (m, l) of up to 64 parts are fetched by one lane each while the O rows
+// of the first parts are already on their way; weights are applied afterwards.
 template <int DT>
 __global__ __launch_bounds__(64) void decode_merge_kernel(void *__restrict__ out,
                                                           const float *__restrict__ part_o,
@@ -342,14 +342,18 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(void *__restrict__ out
                                                           int head_dim)
 {
     typedef LoadElt<DT> L;
+    constexpr int kBatch = 8;   // O rows in flight per round
     const int b = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x;
     const int first = req_parts[2 * b], n = req_parts[2 * b + 1];
     if (n <= 0) return;   // written directly by the attention kernel
     if (first < 0 || first + n > max_slots) return;
+    const float *ml_base = part_ml + ((long)first * n_qo_heads + qh) * 2;
+    const float *o_base = part_o + ((long)first * n_qo_heads + qh) * head_dim;
+    const long ml_stride = (long)n_qo_heads * 2, o_stride = (long)n_qo_heads * head_dim;
     float m = kNegBig;
     for (int s0 = 0; s0 < n; s0 += 64) {
         const int s = s0 + lane;
-        float ms = s < n ? part_ml[((long)(first + s) * n_qo_heads + qh) * 2] : kNegBig;
+        float ms = s < n ? ml_base[s * ml_stride] : kNegBig;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ms = fmaxf(ms, __shfl_xor(ms, o));
         m = fmaxf(m, ms);
@@ -360,19 +364,27 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(void *__restrict__ out
         const int s = s0 + lane;
         float w_lane = 0.f, l_lane = 0.f;
         if (s < n) {
-            const float *ml = part_ml + ((long)(first + s) * n_qo_heads + qh) * 2;
-            w_lane = __builtin_amdgcn_exp2f(ml[0] - m);
-            l_lane = w_lane * ml[1];
+            w_lane = __builtin_amdgcn_exp2f(ml_base[s * ml_stride] - m);
+            l_lane = w_lane * ml_base[s * ml_stride + 1];
         }
         l += wave_sum(l_lane);
         const int cnt = min(64, n - s0);
-        for (int j = 0; j < cnt; j++) {
-            const float w = __shfl(w_lane, j);
-            const float *o = part_o + ((long)(first + s0 + j) * n_qo_heads + qh) * head_dim;
+        for (int j0 = 0; j0 < cnt; j0 += kBatch) {
+            float rows[kBatch][4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int d = lane + 64 * i;
-                if (d < head_dim) acc[i] += w * o[d];
+            for (int j = 0; j < kBatch; j++) {
+                const float *o = o_base + (long)(s0 + min(j0 + j, cnt - 1)) * o_stride;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int d = lane + 64 * i;
+                    rows[j][i] = d < head_dim ? o[d] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kBatch; j++) {
+                const float w = (j0 + j < cnt) ? __shfl(w_lane, min(j0 + j, 63)) : 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[i] += w * rows[j][i];
             }
         }
     }

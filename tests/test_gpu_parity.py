@@ -176,6 +176,29 @@ def test_decode_attention_closed_forms_on_gpu():
     assert max_rel_err(got[1], np.repeat(v, 4, axis=0)) < 2e-2                    # equal keys -> mean V
 
 
+def test_decode_attention_is_bitwise_repeatable_across_launches():
+    """Requests cut across workgroups are merged from partials in slot order: the same
+    plan launched again and again (as for every layer of a step) must give the same bits."""
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+
+    _announce("decode repeatability")
+    lens = [4096, 700, 257, 3000, 16, 5000, 1, 2222]
+    for hq, target in ((32, 0), (64, 37), (32, 8)):
+        sc = make_scenario(34, kv_lens=lens, qo_lens=[1] * len(lens), Hq=hq, dtype="bf16")
+        w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
+        w.begin_forward(_dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                        _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P, target_workgroups=target)
+        q, pages = to_torch(sc.q, "bf16"), to_torch(sc.pages, "bf16")
+        first = w.forward(q, pages).clone()
+        want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                    sc.kv_last_page_lens, "bf16")
+        assert max_rel_err(first.float().cpu().numpy(), want) <= 2e-2
+        outs = [w.forward(q, pages) for _ in range(200)]
+        torch.cuda.synchronize()
+        for i, o in enumerate(outs):
+            assert torch.equal(o.view(torch.int16), first.view(torch.int16)), (hq, target, i)
+
+
 def test_decode_wrapper_protocol_errors():
     from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
 
