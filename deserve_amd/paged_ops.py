@@ -62,6 +62,32 @@ def apply_rope(q: torch.Tensor, k: torch.Tensor, indptr: torch.Tensor, offsets: 
     return q_out, k_out
 
 
+def rope_append_paged_kv_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                               indptr: torch.Tensor, offsets: torch.Tensor,
+                               paged_kv_data: torch.Tensor, kv_indices: torch.Tensor,
+                               kv_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
+                               rope_theta: float = 1e4) -> torch.Tensor:
+    """apply_rope(interleave=True) + append_paged_kv_cache in one kernel: returns the
+    rotated q; the rotated k and v land in their page slots.  Same bits as the two
+    separate calls."""
+    if paged_kv_data.dim() != 5 or paged_kv_data.shape[1] != 2 or not paged_kv_data.is_contiguous():
+        raise ValueError("paged_kv_data must be a contiguous (num_pages, 2, P, Hkv, D) tensor")
+    _, _, P, Hkv, D = paged_kv_data.shape
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    if k.shape != v.shape or tuple(k.shape[1:]) != (Hkv, D) or q.shape[2] != D or \
+            not (q.dtype == k.dtype == v.dtype == paged_kv_data.dtype):
+        raise ValueError("q/k/v must be (nnz, H, D) of the pool's dtype")
+    q_out = torch.empty_like(q)
+    rc = _lib.lib().dskv_rope_append_paged_kv(
+        q_out.data_ptr(), paged_kv_data.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        _i32(indptr).data_ptr(), _i32(offsets).data_ptr(), _i32(kv_indices).data_ptr(),
+        _i32(kv_indptr).data_ptr(), _i32(kv_last_page_len).data_ptr(), indptr.shape[0] - 1,
+        q.shape[0], P, q.shape[1], Hkv, D, float(rope_theta), _lib.dtype_code(q.dtype),
+        _lib.current_stream())
+    _lib.check(rc, "rope_append_paged_kv_cache")
+    return q_out
+
+
 class _PagedWrapper:
     def __init__(self, workspace_buffer: torch.Tensor, kv_layout: str = "NHD") -> None:
         if kv_layout != "NHD":

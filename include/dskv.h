@@ -145,6 +145,20 @@ int dskv_apply_rope(void *q_out, void *k_out, const void *q, const void *k,
                     int32_t dtype, void *stream);
 
 /*
+ * RoPE and KV append in one pass: the two call sites above back to back
+ * (model/layer/attention.py:166-183).  q is rotated into q_out; k is rotated and
+ * written straight into its page slot, v is copied next to it - the rotated K
+ * never makes a round trip through a temporary.  Bit-identical to
+ * dskv_apply_rope followed by dskv_append_paged_kv.
+ */
+int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, const void *q, const void *k,
+                              const void *v, const int32_t *qo_indptr, const int32_t *offsets,
+                              const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
+                              const int32_t *kv_last_page_len, int32_t batch, int32_t nnz,
+                              int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
+                              int32_t head_dim, float rope_theta, int32_t dtype, void *stream);
+
+/*
  * Bulk swap of one contiguous page slice of every layer.  Replaces
  * swap.swap(d, h0, h1, s0, s1, interval) (kvcache/swap.cpp:9-57, called from
  * kvcache/virtual.py:88-95) with the semantics stated by

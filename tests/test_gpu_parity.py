@@ -293,6 +293,27 @@ def test_rope_matches_oracle(dtype):
         apply_rope(to_torch(qs, dtype), to_torch(ks, dtype), _dev_i32(indptr), _dev_i32(offsets))
 
 
+@pytest.mark.parametrize("dtype,P", [("bf16", 16), ("f32", 8), ("f16", 16)])
+def test_fused_rope_append_equals_rope_then_append_bitwise(dtype, P):
+    from deserve_amd.paged_ops import append_paged_kv_cache, apply_rope, rope_append_paged_kv_cache
+
+    _announce("rope+append fused", dtype, P)
+    sc = make_scenario(52, kv_lens=[517, 40, 512, 3, 1029, 77], qo_lens=[512, 40, 1, 3, 0, 1], P=P,
+                       dtype=dtype)
+    offsets = _dev_i32(sc.kv_lens - sc.qo_lens)
+    args = [_dev_i32(x) for x in (sc.kv_page_indices, sc.kv_page_indptr, sc.kv_last_page_lens)]
+    qo = _dev_i32(sc.qo_indptr)
+    q, k, v = (to_torch(x, dtype) for x in (sc.q, sc.k, sc.v))
+    pages_a, pages_b = to_torch(sc.pages, dtype), to_torch(sc.pages, dtype)
+    q_a, k_a = apply_rope(q, k, qo, offsets, interleave=True, rope_theta=5e5)
+    append_paged_kv_cache(k_a, v, qo, pages_a, *args)
+    q_b = rope_append_paged_kv_cache(q, k, v, qo, offsets, pages_b, *args, rope_theta=5e5)
+    torch.cuda.synchronize()
+    assert _same_bits(from_torch(q_a, dtype), from_torch(q_b, dtype))
+    assert _same_bits(from_torch(pages_a, dtype), from_torch(pages_b, dtype))
+    assert not _same_bits(from_torch(pages_a, dtype), sc.pages)
+
+
 # ------------------------------------------------------------------ config 1 of the baseline, exactly
 def test_baseline_config1_fp32_append_then_decode():
     """8 sequences, context 512 after the append, 256-page pool in a seeded random
