@@ -146,8 +146,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void decode_attn_mfma_kernel(
     };
     auto load_next = [&](TileRegs &r) {
         kv.page_ids = cur.page_ids;
-        if (kPageCoversTile) load_kv_tile_in_page(kv, cur.page, cur.t, cur.t_end, g, c, r);
-        else load_kv_tile<false>(kv, cur.t, cur.t_end, g, c, r);
+        if (kPageCoversTile) load_kv_tile_in_page<kLoadStreaming>(kv, cur.page, cur.t, cur.t_end, g, c, r);
+        else load_kv_tile<false, kLoadStreaming>(kv, cur.t, cur.t_end, g, c, r);
         cur.t += kTile;
         settle();
     };

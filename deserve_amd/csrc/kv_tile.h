@@ -21,13 +21,12 @@ constexpr int kVPitch = 288;              // bytes per V row in LDS (256 + 32 pa
 constexpr int kVTileBytes = kTile * kVPitch;
 constexpr int kBufferFlags = 0x00020000;  // raw buffer descriptor word 3 for 32-bit data
 constexpr int kOutOfRange = 0x7FFF0000;   // byte offset no page reaches: reads as zero, moves nothing
-// Cache-policy bits of the K/V stream loads.  Every K/V byte is used once, so the
+// Cache-policy bits of the K/V loads.  Decode uses every K/V byte once, so its
 // loads carry the streaming hint (bit 1): measured on MI355X, a 607 MB read with
-// the hint runs at 6.9 TB/s against 6.3 TB/s without it.
-#ifndef DSKV_KV_LOAD_AUX
-#define DSKV_KV_LOAD_AUX 2
-#endif
-constexpr int kKvLoadAux = DSKV_KV_LOAD_AUX;
+// the hint runs at 6.9 TB/s against 6.3 TB/s without it.  Prefill re-reads each
+// tile from many workgroups and wants it cached, so it loads with policy 0.
+constexpr int kLoadStreaming = 2;
+constexpr int kLoadCached = 0;
 
 // MFMA row m of a tile holds token (m >> 2) + 4 * (m & 3) of that tile.
 __device__ __forceinline__ int row_to_token(int m) { return (m >> 2) + ((m & 3) << 2); }
@@ -60,6 +59,7 @@ struct KvView {
 // rows at or past t_end get an offset outside the page and a tile past the end
 // gets an empty descriptor, so such lanes read zero and generate no memory
 // traffic.  Always issues exactly 8 loads.
+template <int kAux>
 __device__ __forceinline__ void load_kv_tile_in_page(const KvView &kv, long page, int t, int t_end,
                                                      int g, int c, TileRegs &r)
 {
@@ -72,14 +72,14 @@ __device__ __forceinline__ void load_kv_tile_in_page(const KvView &kv, long page
                                        : kOutOfRange;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
-        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, kKvLoadAux);
+        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, kAux);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int vo = (t + g + 4 * i < t_end)
                            ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes + kv.head_off +
                                  c * 16
                            : kOutOfRange;
-        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, kKvLoadAux);
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, kAux);
     }
 }
 
@@ -94,12 +94,12 @@ __device__ __forceinline__ int page_slot_of(const KvView &kv, int t, int t_end)
 // Loads tile [t, t + 16) of a request whose valid tokens end at t_end.  Issued
 // unconditionally (so the count of loads in flight is static); nothing past
 // t_end is fetched.
-template <bool kPageCoversTile>
+template <bool kPageCoversTile, int kAux>
 __device__ __forceinline__ void load_kv_tile(const KvView &kv, int t, int t_end, int g, int c,
                                              TileRegs &r)
 {
     if (kPageCoversTile) {
-        load_kv_tile_in_page(kv, kv.page_ids[page_slot_of(kv, t, t_end)], t, t_end, g, c, r);
+        load_kv_tile_in_page<kAux>(kv, kv.page_ids[page_slot_of(kv, t, t_end)], t, t_end, g, c, r);
     } else {
         // Pages smaller than a tile: every lane resolves its own page.  Tokens
         // past the end are clamped to the last valid one; the consumer masks

@@ -16,8 +16,18 @@
 
 namespace dskv {
 
-constexpr int kPrefillWaves = 8;
-constexpr int kColTiles = 2;   // column tiles (of 16 columns) per wave
+#ifndef DSKV_PREFILL_WAVES
+#define DSKV_PREFILL_WAVES 8
+#endif
+#ifndef DSKV_PREFILL_COLTILES
+#define DSKV_PREFILL_COLTILES 2
+#endif
+#ifndef DSKV_PREFILL_STAGES
+#define DSKV_PREFILL_STAGES 3
+#endif
+constexpr int kPrefillStages = DSKV_PREFILL_STAGES; // tiles in flight per wave
+constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // kv heads per workgroup
+constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 16 columns) per wave
 
 template <int DT, bool kPageCoversTile>
 __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
@@ -61,7 +71,6 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     const bool c_used = c_pos < pos_per_ct;
     int limit[kColTiles];       // number of kv tokens this lane's column may see
     u32x4 qreg[kColTiles][4];
-    int limit_max = 0, limit_min = 0x7FFFFFFF;
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
         const int qrow = q0 + ct * pos_per_ct + c_pos;
@@ -76,16 +85,12 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
             u32x4 z = {0, 0, 0, 0};
             qreg[ct][kk] = live ? *reinterpret_cast<const u32x4 *>(qrow_p + kk * 32) : z;
         }
-        limit_max = max(limit_max, lim);
-        if (live) limit_min = min(limit_min, lim);
     }
-    // wave-wide extremes (lanes of one wave differ in c only; g groups agree)
-#pragma unroll
-    for (int o = 1; o < 16; o <<= 1) {
-        limit_max = max(limit_max, __shfl_xor(limit_max, o));
-        limit_min = min(limit_min, __shfl_xor(limit_min, o));
-    }
-    const int t_end = limit_max;   // uniform: tokens this wave has to walk
+    // Extremes over the tile's live query rows, from scalars only: they steer the
+    // loop and the page lookups and must stay wave-uniform for the compiler too.
+    const int rows_live = min(kColTiles * pos_per_ct, n_b - q0);            // >= 1 by construction
+    const int limit_min = min(max(causal ? kv_len - n_b + q0 + 1 : kv_len, 0), kv_len);
+    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_live : kv_len, 0), kv_len);
 
     f32x4 acc[kColTiles][8];
     float m_run[kColTiles], l_run[kColTiles];
@@ -140,17 +145,28 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         __builtin_amdgcn_wave_barrier();
     };
 
-    // two tile buffers: the next tile loads while the current one is consumed
-    TileRegs ra, rb;
-    load_kv_tile<kPageCoversTile>(kv, 0, t_end, g, c, ra);
-    for (int t = 0; t < t_end; t += 2 * kTile) {
-        load_kv_tile<kPageCoversTile>(kv, t + kTile, t_end, g, c, rb);
-        compute_tile(t, ra);
-        __builtin_amdgcn_sched_barrier(0);
-        load_kv_tile<kPageCoversTile>(kv, t + 2 * kTile, t_end, g, c, ra);
-        if (t + kTile < t_end) compute_tile(t + kTile, rb);
-        __builtin_amdgcn_sched_barrier(0);
+    // A ring of kPrefillStages tile buffers.  The steady-state body is straight
+    // line (loads are unconditional; a tile past the end fetches nothing in the
+    // page-descriptor path), so the compiler waits only for the tile it consumes.
+    TileRegs ring[kPrefillStages];
+    int t = 0;
+#pragma unroll
+    for (int s = 0; s < kPrefillStages; s++)
+        load_kv_tile<kPageCoversTile, kLoadCached>(kv, s * kTile, t_end, g, c, ring[s]);
+    while (t + (kPrefillStages - 1) * kTile < t_end) {
+#pragma unroll
+        for (int s = 0; s < kPrefillStages; s++) {
+            compute_tile(t + s * kTile, ring[s]);
+            __builtin_amdgcn_sched_barrier(0);
+            load_kv_tile<kPageCoversTile, kLoadCached>(kv, t + (s + kPrefillStages) * kTile, t_end, g,
+                                                        c, ring[s]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        t += kPrefillStages * kTile;
     }
+#pragma unroll
+    for (int s = 0; s < kPrefillStages - 1; s++)
+        if (t + s * kTile < t_end) compute_tile(t + s * kTile, ring[s]);
 
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
