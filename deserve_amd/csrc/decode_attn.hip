@@ -174,7 +174,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void decode_attn_mfma_kernel(
         float l_run = 0.f;
 
         auto compute_tile = [&](int t, const TileRegs &r) {
-            // scores: S^T = K . Q^T ; lane holds tokens t + g + 4j of q column c
+            // scores: S^T = K . Q^T ; lane holds tokens t + 4g + j of q column c
             f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < 4; kk++) s = E::mfma_k32(r.k[kk], qreg[kk], s);
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void decode_attn_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 x[j] = s[j] * scale_log2;
-                if (ragged && t + g + 4 * j >= t_end) x[j] = kNegBig;
+                if (ragged && t + 4 * g + j >= t_end) x[j] = kNegBig;
             }
             stage_v_tile<kPageCoversTile>(lds, r, t, t_end, g, c);
             // online softmax (log2 domain)

@@ -2,13 +2,13 @@
 // (head_dim 128, 16-bit elements, one wavefront per kv head).
 //
 // Lane roles, with g = lane / 16 and c = lane % 16:
-//   K: lane holds dims kk*32 + g*8 .. +8 (kk = 0..3) of tile row c, which is
-//      token row_to_token(c) of the tile - the A operand of the 16x16x32 MFMA.
-//   V: lane holds the 16-byte chunk c of tile tokens g, g+4, g+8, g+12; the tile
-//      is written to LDS as loaded and read back column-wise as the A operand of
-//      the 16x16x16 MFMA (4 tokens g, g+4, g+8, g+12 of one dim per lane).
-// The token permutation makes the four lane groups read neighbouring LDS rows of
-// a 288-byte-pitch tile, which is bank-conflict free.
+//   K: lane holds dims kk*32 + g*8 .. +8 (kk = 0..3) of tile token c - the A
+//      operand of the 16x16x32 MFMA, so S^T = K.Q^T has tokens 4g..4g+3 of query
+//      column c in lane (g, c).
+//   V: lane loads the 16-byte chunk c of tile tokens g, g+4, g+8, g+12; the tile
+//      is written to LDS row-major (one token per 288-byte row) and read back
+//      with the transposing LDS read, which hands lane (g, c) tokens 4g..4g+3 of
+//      dim dt*16 + c - the A operand of the P.V MFMA, in the token order S^T has.
 #pragma once
 
 #include "mfma.h"
@@ -20,16 +20,12 @@ constexpr int kHeadDim = 128;             // the MFMA kernels are specialised fo
 constexpr int kVPitch = 288;              // bytes per V row in LDS (256 + 32 pad)
 constexpr int kVTileBytes = kTile * kVPitch;
 constexpr int kBufferFlags = 0x00020000;  // raw buffer descriptor word 3 for 32-bit data
-constexpr int kOutOfRange = 0x7FFF0000;   // byte offset no page reaches: reads as zero, moves nothing
 // Cache-policy bits of the K/V loads.  Decode uses every K/V byte once, so its
 // loads carry the streaming hint (bit 1): measured on MI355X, a 607 MB read with
 // the hint runs at 6.9 TB/s against 6.3 TB/s without it.  Prefill re-reads each
 // tile from many workgroups and wants it cached, so it loads with policy 0.
 constexpr int kLoadStreaming = 2;
 constexpr int kLoadCached = 0;
-
-// MFMA row m of a tile holds token (m >> 2) + 4 * (m & 3) of that tile.
-__device__ __forceinline__ int row_to_token(int m) { return (m >> 2) + ((m & 3) << 2); }
 
 // Block tables and work lists never change while a kernel runs.  Reading them
 // through the constant address space tells the compiler so: wave-uniform reads
@@ -55,31 +51,32 @@ struct KvView {
 };
 
 // Loads tile [t, t + 16), which lies inside pool page `page`, of a request whose
-// valid tokens end at t_end.  The page is addressed through a buffer descriptor:
-// rows at or past t_end get an offset outside the page and a tile past the end
-// gets an empty descriptor, so such lanes read zero and generate no memory
-// traffic.  Always issues exactly 8 loads.
+// valid tokens end at t_end.  The K rows and the V rows of the tile are each
+// addressed through a buffer descriptor that ends after the tile's last valid
+// row: lanes that hold later rows (or a whole tile past the end) read zero and
+// generate no memory traffic, and the per-lane offsets never change.  Always
+// issues exactly 8 loads.
 template <int kAux>
 __device__ __forceinline__ void load_kv_tile_in_page(const KvView &kv, long page, int t, int t_end,
                                                      int g, int c, TileRegs &r)
 {
-    const int k_tok = row_to_token(c);
-    const int slot_off = (t & ((1 << kv.page_shift) - 1)) * kv.row_bytes;
-    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<char *>(kv.pages) + page * kv.page_bytes, 0, t < t_end ? (int)kv.page_bytes : 0,
-        kBufferFlags);
-    const int ko = (t + k_tok < t_end) ? slot_off + k_tok * kv.row_bytes + kv.head_off + g * 16
-                                       : kOutOfRange;
+    const int slot = t & ((1 << kv.page_shift) - 1);
+    // wave-uniform; the clamp would otherwise be selected as a vector instruction
+    const int valid_bytes =
+        __builtin_amdgcn_readfirstlane(min(max(t_end - t, 0), kTile)) * kv.row_bytes;
+    char *first_row = const_cast<char *>(kv.pages) + page * kv.page_bytes + (long)slot * kv.row_bytes;
+    __amdgpu_buffer_rsrc_t k_rows =
+        __builtin_amdgcn_make_buffer_rsrc(first_row, 0, valid_bytes, kBufferFlags);
+    __amdgpu_buffer_rsrc_t v_rows =
+        __builtin_amdgcn_make_buffer_rsrc(first_row + kv.half_bytes, 0, valid_bytes, kBufferFlags);
+    const int ko = c * kv.row_bytes + kv.head_off + g * 16;
 #pragma unroll
     for (int kk = 0; kk < 4; kk++)
-        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ko + kk * 64, 0, kAux);
+        r.k[kk] = __builtin_amdgcn_raw_buffer_load_b128(k_rows, ko + kk * 64, 0, kAux);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int vo = (t + g + 4 * i < t_end)
-                           ? kv.half_bytes + slot_off + (g + 4 * i) * kv.row_bytes + kv.head_off +
-                                 c * 16
-                           : kOutOfRange;
-        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vo, 0, kAux);
+        const int vo = (g + 4 * i) * kv.row_bytes + kv.head_off + c * 16;
+        r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rows, vo, 0, kAux);
     }
 }
 
@@ -104,7 +101,7 @@ __device__ __forceinline__ void load_kv_tile(const KvView &kv, int t, int t_end,
         // Pages smaller than a tile: every lane resolves its own page.  Tokens
         // past the end are clamped to the last valid one; the consumer masks
         // their scores and zeroes their V rows.
-        const int k_tok = row_to_token(c);
+        const int k_tok = c;
         const int page_mask = (1 << kv.page_shift) - 1;
         const int t_last = max(t_end - 1, 0);
         const int tk = min(t + k_tok, t_last);
@@ -144,13 +141,18 @@ __device__ __forceinline__ void stage_v_tile(char *lds, const TileRegs &r, int t
     __builtin_amdgcn_wave_barrier();
 }
 
-// A operand of the P.V MFMA for dim tile dt: V[token g + 4j][dim dt*16 + c], j = 0..3.
+// A operand of the P.V MFMA for dim tile dt: V[token 4g + j][dim dt*16 + c], j = 0..3.
+// The transposing read works on blocks of 16 lanes: lane r of a block supplies
+// the address of four consecutive 16-bit values, and receives value r%4 of the
+// rows supplied by lanes r/4, r/4 + 4, r/4 + 8, r/4 + 12.  Lane (g, r) therefore
+// points at dims dt*16 + 4*(r%4) .. +3 of token 4g + r/4.
+typedef short lds_i16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x2 read_v_operand(const char *lds, int dt, int g, int c)
 {
-    const uint16_t *vc = reinterpret_cast<const uint16_t *>(lds + g * kVPitch) + dt * 16 + c;
-    const uint32_t a0 = vc[0] | ((uint32_t)vc[4 * (kVPitch / 2)] << 16);
-    const uint32_t a1 = vc[8 * (kVPitch / 2)] | ((uint32_t)vc[12 * (kVPitch / 2)] << 16);
-    return u32x2{a0, a1};
+    const char *p = lds + (4 * g + (c >> 2)) * kVPitch + dt * 32 + (c & 3) * 8;
+    const lds_i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) lds_i16x4 *)p);
+    return __builtin_bit_cast(u32x2, v);
 }
 
 }  // namespace dskv

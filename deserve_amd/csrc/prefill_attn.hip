@@ -1,15 +1,19 @@
 // Paged prefill (multi-query) attention with the end-aligned causal mask:
 // query i of the n_b new tokens of request b sees kv positions j <= kv_len_b - n_b + i.
 //
-// Bound: MFMA for long chunks (every K/V tile is reused by all query columns of
-// the wave), L2 for the rest.  Same tile machinery as the decode kernel: K goes
-// HBM/L2 -> VGPR -> MFMA A operand, V is transposed through a wave-private LDS
-// tile, S^T's C layout is reused as the P^T B operand.
+// Bound: MFMA for long chunks.  Work decomposition: one workgroup = one kv head x
+// one tile of query rows; each of its waves owns kColTiles column tiles of 16
+// columns, a column being a (query position, q head of the GQA group) pair, so
+// the MFMA N dimension is dense.  The workgroup walks the request's K/V in
+// blocks of 32 tokens that its waves load together (each a few rows) into a
+// double-buffered LDS stage, so a K/V byte crosses the vector memory path once
+// per workgroup instead of once per wave: with every wave streaming K/V on its
+// own the kernel was bound by that path at a sixth of the MFMA rate.  Per block
+// a wave reads K rows from LDS as the A operand of S^T = K.Q^T, keeps S^T's C
+// layout as the B operand P^T, and reads V through the transposing LDS read.
 //
-// Work decomposition: one wavefront = one kv head x kColTiles column tiles of 16
-// columns.  A column is a (query position, q head of the GQA group) pair, so the
-// MFMA N dimension is dense: 16/group query positions per column tile.  The 8
-// waves of a workgroup are the 8 kv heads of one query tile.
+// Workgroup ids are laid out head-fastest: consecutive ids go to different XCDs,
+// so (with 8 kv heads) all query tiles of one kv head share one XCD's L2.
 #include "kv_tile.h"
 
 #include <algorithm>
@@ -22,14 +26,25 @@ namespace dskv {
 #ifndef DSKV_PREFILL_COLTILES
 #define DSKV_PREFILL_COLTILES 2
 #endif
-#ifndef DSKV_PREFILL_STAGES
-#define DSKV_PREFILL_STAGES 3
-#endif
-constexpr int kPrefillStages = DSKV_PREFILL_STAGES; // tiles in flight per wave
-constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // kv heads per workgroup
+constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
 constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 16 columns) per wave
+constexpr int kBlock = 2 * kTile;                   // tokens per step
+constexpr int kKPitch = 272;                        // bytes per K row in LDS (256 + 16 pad)
+constexpr int kStageK = kBlock * kKPitch;
+constexpr int kStageBytes = kBlock * (kKPitch + kVPitch);
+constexpr int kRowsPerWave = kBlock / kPrefillWaves;   // rows of a block one wave loads
+constexpr int kRowGroups = kRowsPerWave / 4;           // in groups of 4 rows (one load each)
+static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole groups of 4 rows");
+// The running maximum of a column is only raised when a block exceeds it by more
+// than this (log2 domain): probabilities stay below 2^8, the accumulators are
+// rescaled a handful of times per query instead of once per block.
+constexpr float kRescaleSlack = 8.f;
 
-template <int DT, bool kPageCoversTile>
+struct StageRegs {
+    u32x4 k[kRowGroups], v[kRowGroups];
+};
+
+template <int DT, bool kRowsSharePage>
 __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
     const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
@@ -38,34 +53,32 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     int n_kv_heads, int page_shift, float scale_log2, int causal)
 {
     typedef Elt<DT> E;
-    __shared__ __align__(16) char v_lds[kPrefillWaves][kVTileBytes];
+    __shared__ __align__(16) char stage[2][kStageBytes];   // per stage: 32 K rows, 32 V rows
 
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int g = lane >> 4;
     const int c = lane & 15;
-    const int kvh = blockIdx.y * kPrefillWaves + wave;
-    if (kvh >= n_kv_heads) return;
+    const int kvh = blockIdx.x % n_kv_heads;
+    const int tile = blockIdx.x / n_kv_heads;
     const int group = n_qo_heads / n_kv_heads;
-    const int pos_per_ct = 16 / group;            // query positions per column tile
+    const int pos_per_ct = 16 / group;             // query positions per column tile
+    const int pos_per_wave = kColTiles * pos_per_ct;
 
-    const int b = tile_info[2 * blockIdx.x];
-    const int q0 = tile_info[2 * blockIdx.x + 1];   // first query row of the tile within b
+    const int b = tile_info[2 * tile];
+    const int q0 = tile_info[2 * tile + 1];        // first query row of the tile within b
     const int q_begin = qo_indptr[b];
     const int n_b = qo_indptr[b + 1] - q_begin;
     const int n_pages = kv_indptr[b + 1] - kv_indptr[b];
     const int kv_len = n_pages > 0 ? ((n_pages - 1) << page_shift) + kv_last[b] : 0;
+    const_i32_ptr page_ids = as_const(kv_indices) + kv_indptr[b];
+    const int row_bytes = n_kv_heads * kHeadDim * 2;
+    const int half_bytes = row_bytes << page_shift;
+    const long page_bytes = 2L * half_bytes;
+    const int page_mask = (1 << page_shift) - 1;
 
-    KvView kv;
-    kv.pages = pages;
-    kv.page_ids = as_const(kv_indices) + kv_indptr[b];
-    kv.page_shift = page_shift;
-    kv.row_bytes = n_kv_heads * kHeadDim * 2;
-    kv.half_bytes = kv.row_bytes << page_shift;
-    kv.page_bytes = 2L * kv.half_bytes;
-    kv.head_off = kvh * (kHeadDim * 2);
-
-    // column c of column tile ct: query row q0 + ct*pos_per_ct + c/group, head c%group
+    // column c of column tile ct: query row wq0 + ct*pos_per_ct + c/group, head c%group
+    const int wq0 = q0 + wave * pos_per_wave;
     const int c_pos = c / group;
     const int c_head = c - c_pos * group;
     const bool c_used = c_pos < pos_per_ct;
@@ -73,7 +86,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     u32x4 qreg[kColTiles][4];
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
-        const int qrow = q0 + ct * pos_per_ct + c_pos;
+        const int qrow = wq0 + ct * pos_per_ct + c_pos;
         const bool live = c_used && qrow < n_b;
         int lim = causal ? kv_len - n_b + qrow + 1 : kv_len;
         lim = live ? min(max(lim, 0), kv_len) : 0;
@@ -86,94 +99,172 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
             qreg[ct][kk] = live ? *reinterpret_cast<const u32x4 *>(qrow_p + kk * 32) : z;
         }
     }
-    // Extremes over the tile's live query rows, from scalars only: they steer the
-    // loop and the page lookups and must stay wave-uniform for the compiler too.
-    const int rows_live = min(kColTiles * pos_per_ct, n_b - q0);            // >= 1 by construction
-    const int limit_min = min(max(causal ? kv_len - n_b + q0 + 1 : kv_len, 0), kv_len);
-    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_live : kv_len, 0), kv_len);
+    // Token ranges from scalars only: they steer loops, barriers and page lookups
+    // and must be uniform for the compiler too.  The workgroup walks [0, t_end);
+    // a wave computes on [0, w_end) and masks from w_mask_from on.
+    const int rows_wg = min(kPrefillWaves * pos_per_wave, n_b - q0);          // >= 1 by construction
+    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_wg : kv_len, 0), kv_len);
+    const int rows_w = min(pos_per_wave, n_b - wq0);                          // <= 0: idle wave
+    const int w_mask_from =
+        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + 1 : kv_len, 0), kv_len) : 0;
+    const int w_end =
+        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + rows_w : kv_len, 0), kv_len) : 0;
 
+    // Start value of a running maximum: far below any scaled score, far above a
+    // scaled masked score (kNegBig * scale_log2).
+    const float m_floor = 0.5f * kNegBig * scale_log2;
     f32x4 acc[kColTiles][8];
     float m_run[kColTiles], l_run[kColTiles];
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
-        m_run[ct] = kNegBig;
+        m_run[ct] = m_floor;
         l_run[ct] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < 8; dt++) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    char *lds = v_lds[wave];
 
-    auto compute_tile = [&](int t, const TileRegs &r) {
-        stage_v_tile<kPageCoversTile>(lds, r, t, t_end, g, c);
-        const bool need_mask = t + kTile > limit_min;   // wave-uniform
-        u32x2 pb[kColTiles];
-        float alpha[kColTiles];
+    // This wave's share of block [t, t + 32): rows wave*kRowsPerWave .. +kRowsPerWave,
+    // lane (g, c) the 16-byte chunk c of row 4i + g.  Rows at or past t_end read as
+    // zero (their probabilities are zero, but 0 * garbage is not).
+    const int lane_off = g * row_bytes + kvh * (kHeadDim * 2) + c * 16;
+    auto load_rows = [&](int t, StageRegs &r) {
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++) {
+            const int tok0 = t + wave * kRowsPerWave + 4 * i;
+            if (kRowsSharePage) {
+                // one page holds the 4 rows: descriptors that end after the last
+                // valid row make the bounds check free and keep offsets constant
+                const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
+                const int slot = min(tok0 >> page_shift, max((t_end - 1) >> page_shift, 0));
+                const long page = valid > 0 ? page_ids[slot] : 0;   // no lookup past the table
+                char *first_row = const_cast<char *>(pages) + page * page_bytes +
+                                  (long)(tok0 & page_mask) * row_bytes;
+                __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
+                    first_row, 0, valid * row_bytes, kBufferFlags);
+                __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
+                    first_row + half_bytes, 0, valid * row_bytes, kBufferFlags);
+                r.k[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rows, lane_off, 0, kLoadCached);
+                r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rows, lane_off, 0, kLoadCached);
+            } else {
+                const int tok = tok0 + g;
+                const int tc = min(tok, max(t_end - 1, 0));
+                const long page = t_end > 0 ? page_ids[tc >> page_shift] : 0;
+                const char *p = pages + page * page_bytes +
+                                (long)(tc & page_mask) * row_bytes + (lane_off - g * row_bytes);
+                const u32x4 z = {0, 0, 0, 0};
+                const u32x4 kk = *reinterpret_cast<const u32x4 *>(p);
+                const u32x4 vv = *reinterpret_cast<const u32x4 *>(p + half_bytes);
+                r.k[i] = tok < t_end ? kk : z;
+                r.v[i] = tok < t_end ? vv : z;
+            }
+        }
+    };
+    auto store_rows = [&](char *st, const StageRegs &r) {
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++) {
+            const int row = wave * kRowsPerWave + 4 * i + g;
+            *reinterpret_cast<u32x4 *>(st + row * kKPitch + c * 16) = r.k[i];
+            *reinterpret_cast<u32x4 *>(st + kStageK + row * kVPitch + c * 16) = r.v[i];
+        }
+    };
+
+    // One step: 32 tokens against every column of the wave.  S^T (tokens x columns)
+    // comes out of the MFMA with tokens t + 4g + j (low tile) and t + 16 + 4g + j
+    // (high tile) in lane (g, c); packed, those eight probabilities are the B
+    // operand of a 16x16x32 MFMA whose A operand is the matching eight V rows.
+    auto compute_block = [&](int t, const char *st) {
+        const bool need_mask = t + kBlock > w_mask_from;   // wave-uniform
+        const char *k_lo = st + c * kKPitch + g * 16;
+        const char *k_hi = k_lo + kTile * kKPitch;
+        const char *v_lo = st + kStageK;
+        const char *v_hi = v_lo + kTile * kVPitch;
+        u32x4 ka[2][4];
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            ka[0][kk] = *reinterpret_cast<const u32x4 *>(k_lo + kk * 64);
+            ka[1][kk] = *reinterpret_cast<const u32x4 *>(k_hi + kk * 64);
+        }
+        u32x4 pb[kColTiles];
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
-            f32x4 s = {0.f, 0.f, 0.f, 0.f};
+            f32x4 s_lo = {0.f, 0.f, 0.f, 0.f}, s_hi = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) s = E::mfma_k32(r.k[kk], qreg[ct][kk], s);
-            float x[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                x[j] = s[j] * scale_log2;
-                if (need_mask && t + g + 4 * j >= limit[ct]) x[j] = kNegBig;
+            for (int kk = 0; kk < 4; kk++) {
+                s_lo = E::mfma_k32(ka[0][kk], qreg[ct][kk], s_lo);
+                s_hi = E::mfma_k32(ka[1][kk], qreg[ct][kk], s_hi);
             }
-            float m_tile = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32));
-            const float m_new = fmaxf(m_run[ct], m_tile);
-            alpha[ct] = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
-            m_run[ct] = m_new;
-            float p[4], p_sum = 0.f;
+            float x[8];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                // a fully masked column keeps m at kNegBig: force p to 0 there
-                p[j] = x[j] > kNegBig ? __builtin_amdgcn_exp2f(x[j] - m_new) : 0.f;
+                x[j] = s_lo[j];
+                x[4 + j] = s_hi[j];
+            }
+            if (need_mask) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (t + 4 * g + j >= limit[ct]) x[j] = kNegBig;
+                    if (t + kTile + 4 * g + j >= limit[ct]) x[4 + j] = kNegBig;
+                }
+            }
+            // scale_log2 > 0: the maximum can be taken before scaling
+            float m_blk = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                                fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+            m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16));
+            m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
+            m_blk *= scale_log2;
+            if (__builtin_amdgcn_ballot_w64(m_blk > m_run[ct] + kRescaleSlack) != 0) {
+                const float m_new = fmaxf(m_run[ct], m_blk);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
+                m_run[ct] = m_new;
+                l_run[ct] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < 8; dt++) acc[ct][dt] *= alpha;
+            }
+            // a masked score is kNegBig and m_run never drops below m_floor, so
+            // masked probabilities come out as exp2(-huge) = 0 without a select
+            float p[8], p_sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[j], scale_log2, -m_run[ct]));
                 p_sum += p[j];
             }
-            l_run[ct] = l_run[ct] * alpha[ct] + p_sum;
-            pb[ct] = u32x2{E::pack2(p[0], p[1]), E::pack2(p[2], p[3])};
+            l_run[ct] += p_sum;
+            pb[ct] = u32x4{E::pack2(p[0], p[1]), E::pack2(p[2], p[3]), E::pack2(p[4], p[5]),
+                           E::pack2(p[6], p[7])};
         }
 #pragma unroll
         for (int dt = 0; dt < 8; dt++) {
-            const u32x2 va = read_v_operand(lds, dt, g, c);
+            const u32x2 a_lo = read_v_operand(v_lo, dt, g, c);
+            const u32x2 a_hi = read_v_operand(v_hi, dt, g, c);
+            const u32x4 va = {a_lo.x, a_lo.y, a_hi.x, a_hi.y};
 #pragma unroll
-            for (int ct = 0; ct < kColTiles; ct++)
-                acc[ct][dt] = E::mfma_k16(va, pb[ct], acc[ct][dt] * alpha[ct]);
+            for (int ct = 0; ct < kColTiles; ct++) acc[ct][dt] = E::mfma_k32(va, pb[ct], acc[ct][dt]);
         }
-        __builtin_amdgcn_wave_barrier();
     };
 
-    // A ring of kPrefillStages tile buffers.  The steady-state body is straight
-    // line (loads are unconditional; a tile past the end fetches nothing in the
-    // page-descriptor path), so the compiler waits only for the tile it consumes.
-    TileRegs ring[kPrefillStages];
-    int t = 0;
-#pragma unroll
-    for (int s = 0; s < kPrefillStages; s++)
-        load_kv_tile<kPageCoversTile, kLoadCached>(kv, s * kTile, t_end, g, c, ring[s]);
-    while (t + (kPrefillStages - 1) * kTile < t_end) {
-#pragma unroll
-        for (int s = 0; s < kPrefillStages; s++) {
-            compute_tile(t + s * kTile, ring[s]);
-            __builtin_amdgcn_sched_barrier(0);
-            load_kv_tile<kPageCoversTile, kLoadCached>(kv, t + (s + kPrefillStages) * kTile, t_end, g,
-                                                        c, ring[s]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        t += kPrefillStages * kTile;
+    // Block n is computed from stage n % 2 while block n + 1 is written to the
+    // other stage and block n + 2 is on its way from memory.  One barrier per
+    // block: past it every wave has finished reading the stage about to be
+    // overwritten and has finished writing the stage about to be read.  Every
+    // wave runs every iteration (idle ones only load), so the barriers match.
+    StageRegs regs;
+    load_rows(0, regs);
+    store_rows(stage[0], regs);
+    load_rows(kBlock, regs);
+    for (int t = 0; t < t_end; t += kBlock) {
+        const int cur = (t / kBlock) & 1;
+        __syncthreads();
+        store_rows(stage[cur ^ 1], regs);
+        load_rows(t + 2 * kBlock, regs);
+        if (t < w_end) compute_block(t, stage[cur]);
     }
-#pragma unroll
-    for (int s = 0; s < kPrefillStages - 1; s++)
-        if (t + s * kTile < t_end) compute_tile(t + s * kTile, ring[s]);
 
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
         float l = l_run[ct];
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
-        const int qrow = q0 + ct * pos_per_ct + c_pos;
+        const int qrow = wq0 + ct * pos_per_ct + c_pos;
         if (!(c_used && qrow < n_b)) continue;
         const float inv = l > 0.f ? 1.f / l : 0.f;
         uint16_t *o = out + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim +
@@ -257,7 +348,7 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
 static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads)
 {
     const int group = n_qo_heads / n_kv_heads;
-    return group <= 16 ? kColTiles * (16 / group) : 1;
+    return group <= 16 ? kPrefillWaves * kColTiles * (16 / group) : 1;
 }
 
 }  // namespace dskv
@@ -327,28 +418,29 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     DSKV_REQUIRE(n_qo_heads <= 65535, "prefill_attn: too many heads");
     const float scale_log2 = sm_scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
+    // the MFMA kernel takes maxima before scaling: it needs a positive, sane scale
     const bool mfma = (dtype == DSKV_BF16 || dtype == DSKV_F16) && head_dim == kHeadDim &&
-                      n_qo_heads / n_kv_heads <= 16;
+                      n_qo_heads / n_kv_heads <= 16 && scale_log2 > 1e-6f && scale_log2 < 1e6f;
     if (mfma) {
         DSKV_REQUIRE(tile_info_dev && n_tiles > 0, "prefill_attn: missing tile list");
         DSKV_REQUIRE(((uintptr_t)out | (uintptr_t)q | (uintptr_t)pages_layer) % 16 == 0,
                      "prefill_attn: out/q/pages must be 16-byte aligned");
         DSKV_REQUIRE(is_pow2(page_size),
                      "prefill_attn: 16-bit path needs a power-of-two page size, got %d", page_size);
-        const int waves = std::min(n_kv_heads, kPrefillWaves);
-        dim3 grid((unsigned)n_tiles, (unsigned)((n_kv_heads + kPrefillWaves - 1) / kPrefillWaves));
-        dim3 block(64 * waves);
+        DSKV_REQUIRE((int64_t)n_tiles * n_kv_heads < (int64_t(1) << 31), "prefill_attn: too many tiles");
+        dim3 grid((unsigned)n_tiles * (unsigned)n_kv_heads);
+        dim3 block(64 * kPrefillWaves);
         const int shift = ilog2(page_size);
-#define DSKV_LAUNCH_PREFILL(DT, COVER)                                                          \
-    hipLaunchKernelGGL((prefill_attn_mfma_kernel<DT, COVER>), grid, block, 0, s, (uint16_t *)out, \
+#define DSKV_LAUNCH_PREFILL(DT, SHARE)                                                          \
+    hipLaunchKernelGGL((prefill_attn_mfma_kernel<DT, SHARE>), grid, block, 0, s, (uint16_t *)out, \
                        (const uint16_t *)q, qo_indptr, (const char *)pages_layer,               \
                        kv_page_indices, kv_page_indptr, kv_last_page_len, tile_info_dev,        \
                        n_qo_heads, n_kv_heads, shift, scale_log2, causal)
         if (dtype == DSKV_BF16) {
-            if (page_size >= kTile) DSKV_LAUNCH_PREFILL(DSKV_BF16, true);
+            if (page_size >= 4) DSKV_LAUNCH_PREFILL(DSKV_BF16, true);
             else DSKV_LAUNCH_PREFILL(DSKV_BF16, false);
         } else {
-            if (page_size >= kTile) DSKV_LAUNCH_PREFILL(DSKV_F16, true);
+            if (page_size >= 4) DSKV_LAUNCH_PREFILL(DSKV_F16, true);
             else DSKV_LAUNCH_PREFILL(DSKV_F16, false);
         }
 #undef DSKV_LAUNCH_PREFILL
