@@ -141,18 +141,23 @@ __device__ __forceinline__ void stage_v_tile(char *lds, const TileRegs &r, int t
     __builtin_amdgcn_wave_barrier();
 }
 
-// A operand of the P.V MFMA for dim tile dt: V[token 4g + j][dim dt*16 + c], j = 0..3.
-// The transposing read works on blocks of 16 lanes: lane r of a block supplies
-// the address of four consecutive 16-bit values, and receives value r%4 of the
-// rows supplied by lanes r/4, r/4 + 4, r/4 + 8, r/4 + 12.  Lane (g, r) therefore
-// points at dims dt*16 + 4*(r%4) .. +3 of token 4g + r/4.
+// The transposing LDS read works on blocks of 16 lanes: lane i of a block
+// supplies the address of four consecutive 16-bit values ("its row"), and
+// receives value i%4 of the rows supplied by lanes i/4, i/4 + 4, i/4 + 8 and
+// i/4 + 12 of its block.
 typedef short lds_i16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 read_transposed(const char *row)
+{
+    const lds_i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) lds_i16x4 *)row);
+    return __builtin_bit_cast(u32x2, v);
+}
+
+// A operand of the 16x16x16 P.V MFMA for dim tile dt: V[token 4g + j][dim dt*16 + c],
+// j = 0..3.  Lane (g, i) points at dims dt*16 + 4*(i%4) .. +3 of token 4g + i/4.
 __device__ __forceinline__ u32x2 read_v_operand(const char *lds, int dt, int g, int c)
 {
-    const char *p = lds + (4 * g + (c >> 2)) * kVPitch + dt * 32 + (c & 3) * 8;
-    const lds_i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) lds_i16x4 *)p);
-    return __builtin_bit_cast(u32x2, v);
+    return read_transposed(lds + (4 * g + (c >> 2)) * kVPitch + dt * 32 + (c & 3) * 8);
 }
 
 }  // namespace dskv

@@ -21,6 +21,10 @@ template <> struct Elt<DSKV_BF16> {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8, a),
                                                         __builtin_bit_cast(v8, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x16 mfma_32x32(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8, a),
+                                                        __builtin_bit_cast(v8, b), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ f32x4 mfma_k16(u32x2 a, u32x2 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(v4, a),
                                                           __builtin_bit_cast(v4, b), c, 0, 0, 0);
@@ -31,6 +35,10 @@ template <> struct Elt<DSKV_BF16> {
     }
     static __device__ __forceinline__ float widen(uint16_t h) {
         return __builtin_bit_cast(float, (uint32_t)h << 16);
+    }
+    static __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+        lo = __builtin_bit_cast(float, w << 16);
+        hi = __builtin_bit_cast(float, w & 0xFFFF0000u);
     }
 };
 
@@ -43,6 +51,10 @@ template <> struct Elt<DSKV_F16> {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8, a),
                                                        __builtin_bit_cast(v8, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x16 mfma_32x32(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8, a),
+                                                       __builtin_bit_cast(v8, b), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ f32x4 mfma_k16(u32x2 a, u32x2 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(v4, a),
                                                       __builtin_bit_cast(v4, b), c, 0, 0, 0);
@@ -53,6 +65,11 @@ template <> struct Elt<DSKV_F16> {
     }
     static __device__ __forceinline__ float widen(uint16_t h) {
         return (float)__builtin_bit_cast(_Float16, h);
+    }
+    static __device__ __forceinline__ void unpack2(uint32_t w, float &lo, float &hi) {
+        const v2 h = __builtin_bit_cast(v2, w);
+        lo = (float)h.x;
+        hi = (float)h.y;
     }
 };
 
@@ -79,6 +96,36 @@ template <> struct LoadElt<DSKV_BF16> {
         ((__bf16 *)p)[i] = (__bf16)v;
     }
 };
+
+// Exchange between the four lanes that share lane % 16 (lane bits 4 and 5) with
+// gfx950's register swaps: after swap_rows16(a, b) on a == b == v, a and b hold
+// v of the two lanes that differ in bit 4 (swap_halves32: bit 5).  Pure VALU,
+// where __shfl_xor would go through the LDS pipeline.  The s_nop covers the
+// wait states the swap needs after a vector write of its operands.
+__device__ __forceinline__ void swap_rows16(float &a, float &b)
+{
+    asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_halves32(float &a, float &b)
+{
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float quad_rows_max(float v)
+{
+    float a = v, b = v;
+    swap_rows16(a, b);
+    a = b = fmaxf(a, b);
+    swap_halves32(a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float quad_rows_sum(float v)
+{
+    float a = v, b = v;
+    swap_rows16(a, b);
+    a = b = a + b;
+    swap_halves32(a, b);
+    return a + b;
+}
 
 __device__ __forceinline__ float wave_sum(float v)
 {

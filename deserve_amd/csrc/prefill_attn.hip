@@ -2,15 +2,19 @@
 // query i of the n_b new tokens of request b sees kv positions j <= kv_len_b - n_b + i.
 //
 // Bound: MFMA for long chunks.  Work decomposition: one workgroup = one kv head x
-// one tile of query rows; each of its waves owns kColTiles column tiles of 16
-// columns, a column being a (query position, q head of the GQA group) pair, so
-// the MFMA N dimension is dense.  The workgroup walks the request's K/V in
-// blocks of 32 tokens that its waves load together (each a few rows) into a
-// double-buffered LDS stage, so a K/V byte crosses the vector memory path once
-// per workgroup instead of once per wave: with every wave streaming K/V on its
-// own the kernel was bound by that path at a sixth of the MFMA rate.  Per block
-// a wave reads K rows from LDS as the A operand of S^T = K.Q^T, keeps S^T's C
-// layout as the B operand P^T, and reads V through the transposing LDS read.
+// one tile of query rows; each of its waves owns 32 columns, a column being a
+// (query position, q head of the GQA group) pair, so the MFMA N dimension is
+// dense.  The workgroup walks the request's K/V in blocks of 32 tokens that its
+// waves load together (each a few rows) into a double-buffered LDS stage, so a
+// K/V byte crosses the vector memory path once per workgroup instead of once per
+// wave: with every wave streaming K/V on its own the kernel was bound by that
+// path at a sixth of the MFMA rate.
+//
+// All products use the 32x32x16 MFMA (measured on MI355X at 2.2 PFLOP/s bf16,
+// against 1.3 PFLOP/s for 16x16x32).  Per block a wave computes S^T = K.Q^T
+// (tokens x columns, K rows from LDS as the A operand), keeps S^T's C layout as
+// the B operand P^T, and reads V through the transposing LDS read as the A
+// operand of O^T += V^T.P^T.
 //
 // Workgroup ids are laid out head-fastest: consecutive ids go to different XCDs,
 // so (with 8 kv heads) all query tiles of one kv head share one XCD's L2.
@@ -23,15 +27,17 @@ namespace dskv {
 #ifndef DSKV_PREFILL_WAVES
 #define DSKV_PREFILL_WAVES 8
 #endif
-#ifndef DSKV_PREFILL_COLTILES
-#define DSKV_PREFILL_COLTILES 2
+#ifndef DSKV_PREFILL_KPITCH
+#define DSKV_PREFILL_KPITCH 272
+#endif
+#ifndef DSKV_PREFILL_VPITCH
+#define DSKV_PREFILL_VPITCH 320
 #endif
 constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
-constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 16 columns) per wave
-constexpr int kBlock = 2 * kTile;                   // tokens per step
-constexpr int kKPitch = 272;                        // bytes per K row in LDS (256 + 16 pad)
-constexpr int kStageK = kBlock * kKPitch;
-constexpr int kStageBytes = kBlock * (kKPitch + kVPitch);
+constexpr int kWaveCols = 32;                       // columns per wave (one MFMA tile)
+constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
+constexpr int kKPitch = DSKV_PREFILL_KPITCH;        // bytes per K row in LDS (256 + pad)
+constexpr int kPVPitch = DSKV_PREFILL_VPITCH;       // bytes per V row in LDS (256 + pad)
 constexpr int kRowsPerWave = kBlock / kPrefillWaves;   // rows of a block one wave loads
 constexpr int kRowGroups = kRowsPerWave / 4;           // in groups of 4 rows (one load each)
 static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole groups of 4 rows");
@@ -40,10 +46,9 @@ static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole grou
 // rescaled a handful of times per query instead of once per block.
 constexpr float kRescaleSlack = 8.f;
 
-struct StageRegs {
-    u32x4 k[kRowGroups], v[kRowGroups];
-};
-
+// Lane roles of the 32x32x16 MFMA, with h = lane / 32 and r = lane % 32:
+//   A operand: row r, k = 8h .. 8h+7.   B operand: column r, k = 8h .. 8h+7.
+//   C/D: column r, rows 8i + 4h + j in register 4i + j (i, j = 0..3).
 template <int DT, bool kRowsSharePage>
 __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
@@ -53,17 +58,19 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     int n_kv_heads, int page_shift, float scale_log2, int causal)
 {
     typedef Elt<DT> E;
-    __shared__ __align__(16) char stage[2][kStageBytes];   // per stage: 32 K rows, 32 V rows
+    __shared__ __align__(16) char k_stage[3][kBlock * kKPitch];
+    __shared__ __align__(16) char v_stage[2][kBlock * kPVPitch];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    const int g = lane >> 4;
+    const int g = lane >> 4;     // row group / chunk roles of the K/V row movement
     const int c = lane & 15;
+    const int h = lane >> 5;     // MFMA roles
+    const int r = lane & 31;
     const int kvh = blockIdx.x % n_kv_heads;
     const int tile = blockIdx.x / n_kv_heads;
     const int group = n_qo_heads / n_kv_heads;
-    const int pos_per_ct = 16 / group;             // query positions per column tile
-    const int pos_per_wave = kColTiles * pos_per_ct;
+    const int pos_per_wave = kWaveCols / group;    // query positions per wave
 
     const int b = tile_info[2 * tile];
     const int q0 = tile_info[2 * tile + 1];        // first query row of the tile within b
@@ -77,26 +84,22 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     const long page_bytes = 2L * half_bytes;
     const int page_mask = (1 << page_shift) - 1;
 
-    // column c of column tile ct: query row wq0 + ct*pos_per_ct + c/group, head c%group
+    // column r: query row wq0 + r/group, head r%group
     const int wq0 = q0 + wave * pos_per_wave;
-    const int c_pos = c / group;
-    const int c_head = c - c_pos * group;
-    const bool c_used = c_pos < pos_per_ct;
-    int limit[kColTiles];       // number of kv tokens this lane's column may see
-    u32x4 qreg[kColTiles][4];
-#pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        const int qrow = wq0 + ct * pos_per_ct + c_pos;
-        const bool live = c_used && qrow < n_b;
-        int lim = causal ? kv_len - n_b + qrow + 1 : kv_len;
-        lim = live ? min(max(lim, 0), kv_len) : 0;
-        limit[ct] = lim;
+    const int c_pos = r / group;
+    const int c_head = r - c_pos * group;
+    const int qrow = wq0 + c_pos;
+    const bool live = c_pos < pos_per_wave && qrow < n_b;
+    int limit = causal ? kv_len - n_b + qrow + 1 : kv_len;   // kv tokens this column may see
+    limit = live ? min(max(limit, 0), kv_len) : 0;
+    u32x4 qreg[8];     // dims 16*ks + 8h .. +7 of the column's query
+    {
         const uint16_t *qrow_p =
-            q + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim + g * 8;
+            q + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim + h * 8;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
+        for (int ks = 0; ks < 8; ks++) {
             u32x4 z = {0, 0, 0, 0};
-            qreg[ct][kk] = live ? *reinterpret_cast<const u32x4 *>(qrow_p + kk * 32) : z;
+            qreg[ks] = live ? *reinterpret_cast<const u32x4 *>(qrow_p + ks * 16) : z;
         }
     }
     // Token ranges from scalars only: they steer loops, barriers and page lookups
@@ -110,171 +113,283 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     const int w_end =
         rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + rows_w : kv_len, 0), kv_len) : 0;
 
-    // Start value of a running maximum: far below any scaled score, far above a
+    const int n_blocks = (t_end + kBlock - 1) / kBlock;
+    // Start value of the running maximum: far below any scaled score, far above a
     // scaled masked score (kNegBig * scale_log2).
-    const float m_floor = 0.5f * kNegBig * scale_log2;
-    f32x4 acc[kColTiles][8];
-    float m_run[kColTiles], l_run[kColTiles];
+    float m_run = 0.5f * kNegBig * scale_log2, l_run = 0.f;
+    f32x16 acc[4];     // O^T: dims 32*dt + 8i + 4h + j of column r in acc[dt][4i + j]
+    u32x4 pb[2];       // packed probabilities of the previous block, per k-step
 #pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        m_run[ct] = m_floor;
-        l_run[ct] = 0.f;
+    for (int dt = 0; dt < 4; dt++)
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int v = 0; v < 16; v++) acc[dt][v] = 0.f;
+    pb[0] = pb[1] = u32x4{0, 0, 0, 0};
+
+    // No kv token visible to any row of the tile: the output rows are zero.
+    // (Uniform over the workgroup, and before the first barrier.)
+    if (t_end == 0) {
+        if (live) {
+            uint16_t *o = out + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim +
+                          4 * h;
+#pragma unroll
+            for (int i = 0; i < 16; i++) *reinterpret_cast<u32x2 *>(o + 8 * i) = u32x2{0, 0};
+        }
+        return;
     }
 
-    // This wave's share of block [t, t + 32): rows wave*kRowsPerWave .. +kRowsPerWave,
-    // lane (g, c) the 16-byte chunk c of row 4i + g.  Rows at or past t_end read as
-    // zero (their probabilities are zero, but 0 * garbage is not).
+    // This wave's share of the K (or V) rows of block blk: rows
+    // wave*kRowsPerWave .. +kRowsPerWave, lane (g, c) the 16-byte chunk c of row
+    // 4i + g.  Rows at or past t_end read as zero (their probabilities are zero,
+    // but 0 * garbage is not).  Page ids are looked up with a vector load (every
+    // lane the same entry; entries past the table read as page 0, whose
+    // descriptor is then empty): vector loads return in order, so waiting for an
+    // LDS read does not have to wait for these too, as it would for a scalar load.
     const int lane_off = g * row_bytes + kvh * (kHeadDim * 2) + c * 16;
-    auto load_rows = [&](int t, StageRegs &r) {
+    __amdgpu_buffer_rsrc_t page_table = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int32_t *>(kv_indices + kv_indptr[b]), 0, n_pages * 4, kBufferFlags);
+    auto lookup_pages = [&](int blk, int(&pg)[kRowGroups]) {
+        if (!kRowsSharePage) return;
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
-            const int tok0 = t + wave * kRowsPerWave + 4 * i;
+            const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
+            pg[i] = __builtin_amdgcn_raw_buffer_load_b32(page_table, (tok0 >> page_shift) * 4 + lane * 0, 0, 0);
+        }
+    };
+    auto load_rows = [&](int blk, int half_off, const int(&pg)[kRowGroups], u32x4(&rows)[kRowGroups]) {
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++) {
+            const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
             if (kRowsSharePage) {
-                // one page holds the 4 rows: descriptors that end after the last
-                // valid row make the bounds check free and keep offsets constant
+                // one page holds the 4 rows: a descriptor that ends after the last
+                // valid row makes the bounds check free and keeps offsets constant
                 const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
-                const int slot = min(tok0 >> page_shift, max((t_end - 1) >> page_shift, 0));
-                const long page = valid > 0 ? page_ids[slot] : 0;   // no lookup past the table
-                char *first_row = const_cast<char *>(pages) + page * page_bytes +
+                const long page = __builtin_amdgcn_readfirstlane(pg[i]);
+                char *first_row = const_cast<char *>(pages) + page * page_bytes + half_off +
                                   (long)(tok0 & page_mask) * row_bytes;
-                __amdgpu_buffer_rsrc_t k_rows = __builtin_amdgcn_make_buffer_rsrc(
+                __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc(
                     first_row, 0, valid * row_bytes, kBufferFlags);
-                __amdgpu_buffer_rsrc_t v_rows = __builtin_amdgcn_make_buffer_rsrc(
-                    first_row + half_bytes, 0, valid * row_bytes, kBufferFlags);
-                r.k[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rows, lane_off, 0, kLoadCached);
-                r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rows, lane_off, 0, kLoadCached);
+                rows[i] = __builtin_amdgcn_raw_buffer_load_b128(desc, lane_off, 0, kLoadCached);
             } else {
                 const int tok = tok0 + g;
-                const int tc = min(tok, max(t_end - 1, 0));
-                const long page = t_end > 0 ? page_ids[tc >> page_shift] : 0;
-                const char *p = pages + page * page_bytes +
+                const int tc = min(tok, t_end - 1);
+                const char *p = pages + page_ids[tc >> page_shift] * page_bytes + half_off +
                                 (long)(tc & page_mask) * row_bytes + (lane_off - g * row_bytes);
                 const u32x4 z = {0, 0, 0, 0};
-                const u32x4 kk = *reinterpret_cast<const u32x4 *>(p);
-                const u32x4 vv = *reinterpret_cast<const u32x4 *>(p + half_bytes);
-                r.k[i] = tok < t_end ? kk : z;
-                r.v[i] = tok < t_end ? vv : z;
+                const u32x4 got = *reinterpret_cast<const u32x4 *>(p);
+                rows[i] = tok < t_end ? got : z;
             }
         }
     };
-    auto store_rows = [&](char *st, const StageRegs &r) {
+    auto store_rows = [&](char *st, int pitch, const u32x4(&rows)[kRowGroups]) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
             const int row = wave * kRowsPerWave + 4 * i + g;
-            *reinterpret_cast<u32x4 *>(st + row * kKPitch + c * 16) = r.k[i];
-            *reinterpret_cast<u32x4 *>(st + kStageK + row * kVPitch + c * 16) = r.v[i];
+            *reinterpret_cast<u32x4 *>(st + row * pitch + c * 16) = rows[i];
         }
     };
 
-    // One step: 32 tokens against every column of the wave.  S^T (tokens x columns)
-    // comes out of the MFMA with tokens t + 4g + j (low tile) and t + 16 + 4g + j
-    // (high tile) in lane (g, c); packed, those eight probabilities are the B
-    // operand of a 16x16x32 MFMA whose A operand is the matching eight V rows.
-    auto compute_block = [&](int t, const char *st) {
-        const bool need_mask = t + kBlock > w_mask_from;   // wave-uniform
-        const char *k_lo = st + c * kKPitch + g * 16;
-        const char *k_hi = k_lo + kTile * kKPitch;
-        const char *v_lo = st + kStageK;
-        const char *v_hi = v_lo + kTile * kVPitch;
-        u32x4 ka[2][4];
+    // S^T = K.Q^T of one block, unscaled: tokens 8i + 4h + j of column r in
+    // x[4i + j].  Registers 8s .. 8s+7, packed, are the B operand of the P.V MFMA
+    // for k-step s, which thereby fixes the tokens of that step's k slots:
+    // 16s + 4h + j in slots j, 16s + 8 + 4h + j in slots 4 + j.
+    float x[16];
+    u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
+    auto read_k_operands = [&](const char *kst) {
+        const char *k_rows = kst + r * kKPitch + h * 16;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            ka[0][kk] = *reinterpret_cast<const u32x4 *>(k_lo + kk * 64);
-            ka[1][kk] = *reinterpret_cast<const u32x4 *>(k_hi + kk * 64);
-        }
-        u32x4 pb[kColTiles];
+        for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 32);
+    };
+    auto scores = [&]() {
+        f32x16 s;
 #pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            f32x4 s_lo = {0.f, 0.f, 0.f, 0.f}, s_hi = {0.f, 0.f, 0.f, 0.f};
+        for (int v = 0; v < 16; v++) s[v] = 0.f;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                s_lo = E::mfma_k32(ka[0][kk], qreg[ct][kk], s_lo);
-                s_hi = E::mfma_k32(ka[1][kk], qreg[ct][kk], s_hi);
-            }
-            float x[8];
+        for (int ks = 0; ks < 8; ks++) s = E::mfma_32x32(ka[ks], qreg[ks], s);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                x[j] = s_lo[j];
-                x[4 + j] = s_hi[j];
-            }
-            if (need_mask) {
+        for (int v = 0; v < 16; v++) x[v] = s[v];
+    };
+    // Masks block blk's scores (needed from w_mask_from on).
+    auto mask_scores = [&](int blk) {
+        const int t = blk * kBlock;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    if (t + 4 * g + j >= limit[ct]) x[j] = kNegBig;
-                    if (t + kTile + 4 * g + j >= limit[ct]) x[4 + j] = kNegBig;
-                }
-            }
-            // scale_log2 > 0: the maximum can be taken before scaling
-            float m_blk = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
-                                fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-            m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16));
-            m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32));
-            m_blk *= scale_log2;
-            if (__builtin_amdgcn_ballot_w64(m_blk > m_run[ct] + kRescaleSlack) != 0) {
-                const float m_new = fmaxf(m_run[ct], m_blk);
-                const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
-                m_run[ct] = m_new;
-                l_run[ct] *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < 8; dt++) acc[ct][dt] *= alpha;
-            }
-            // a masked score is kNegBig and m_run never drops below m_floor, so
-            // masked probabilities come out as exp2(-huge) = 0 without a select
-            float p[8], p_sum = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                p[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[j], scale_log2, -m_run[ct]));
-                p_sum += p[j];
-            }
-            l_run[ct] += p_sum;
-            pb[ct] = u32x4{E::pack2(p[0], p[1]), E::pack2(p[2], p[3]), E::pack2(p[4], p[5]),
-                           E::pack2(p[6], p[7])};
-        }
-#pragma unroll
-        for (int dt = 0; dt < 8; dt++) {
-            const u32x2 a_lo = read_v_operand(v_lo, dt, g, c);
-            const u32x2 a_hi = read_v_operand(v_hi, dt, g, c);
-            const u32x4 va = {a_lo.x, a_lo.y, a_hi.x, a_hi.y};
-#pragma unroll
-            for (int ct = 0; ct < kColTiles; ct++) acc[ct][dt] = E::mfma_k32(va, pb[ct], acc[ct][dt]);
-        }
+        for (int v = 0; v < 16; v++)
+            if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit) x[v] = kNegBig;
+    };
+    // Column maximum of the block in x, and whether the running maximum has to be
+    // raised before the block's exponentials.
+    float m_blk = 0.f;
+    bool raise = false;
+    auto block_max = [&]() {
+        // scale_log2 > 0: the maximum can be taken before scaling
+        float m = fmaxf(fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
+                              fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]))),
+                        fmaxf(fmaxf(fmaxf(x[8], x[9]), fmaxf(x[10], x[11])),
+                              fmaxf(fmaxf(x[12], x[13]), fmaxf(x[14], x[15]))));
+        float other = m;
+        swap_halves32(m, other);
+        m_blk = fmaxf(m, other) * scale_log2;
+        raise = m_blk > m_run + kRescaleSlack;
     };
 
-    // Block n is computed from stage n % 2 while block n + 1 is written to the
-    // other stage and block n + 2 is on its way from memory.  One barrier per
-    // block: past it every wave has finished reading the stage about to be
-    // overwritten and has finished writing the stage about to be read.  Every
-    // wave runs every iteration (idle ones only load), so the barriers match.
-    StageRegs regs;
-    load_rows(0, regs);
-    store_rows(stage[0], regs);
-    load_rows(kBlock, regs);
-    for (int t = 0; t < t_end; t += kBlock) {
-        const int cur = (t / kBlock) & 1;
+    // The K rows run two blocks ahead of the V rows: iteration m of the main loop
+    // multiplies P(m-1) into V(m-1), turns S(m) into P(m) and computes S(m+1), so
+    // that every MFMA of the iteration is independent of its exponentials and the
+    // matrix and vector pipelines of a wave overlap.  Per iteration one barrier:
+    // past it K(m+2) and V(m-1) are complete, and the stages that held K(m) and
+    // V(m-2) are free for K(m+3) and V(m).  Every wave runs every iteration (idle
+    // ones only move rows), so the barriers match.
+    struct RowSet {
+        u32x4 k[kRowGroups], v[kRowGroups];       // rows on their way to LDS
+        int k_pg[kRowGroups], v_pg[kRowGroups];   // page ids of the rows requested next
+    };
+    RowSet even, odd;
+    {
+        int pg[kRowGroups];
+        u32x4 first[3][kRowGroups];
+#pragma unroll
+        for (int blk = 0; blk < 3; blk++) {
+            lookup_pages(blk, pg);
+            load_rows(blk, 0, pg, first[blk]);
+        }
+        const u32x4 z = {0, 0, 0, 0};
+        u32x4 zero[kRowGroups];
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++) zero[i] = z;
+        store_rows(v_stage[1], kPVPitch, zero);   // V(-1): multiplied by P(-1) = 0, must be finite
+#pragma unroll
+        for (int blk = 0; blk < 3; blk++) store_rows(k_stage[blk], kKPitch, first[blk]);
+    }
+    lookup_pages(3, even.k_pg);
+    lookup_pages(4, odd.k_pg);
+    lookup_pages(0, even.v_pg);
+    lookup_pages(1, odd.v_pg);
+    load_rows(3, 0, even.k_pg, even.k);
+    load_rows(4, 0, odd.k_pg, odd.k);
+    load_rows(0, half_bytes, even.v_pg, even.v);
+    load_rows(1, half_bytes, odd.v_pg, odd.v);
+    lookup_pages(5, even.k_pg);
+    lookup_pages(6, odd.k_pg);
+    lookup_pages(2, even.v_pg);
+    lookup_pages(3, odd.v_pg);
+    __syncthreads();
+    if (w_end > 0) {
+        read_k_operands(k_stage[0]);
+        scores();
+        if (kBlock > w_mask_from) mask_scores(0);
+        block_max();
+        read_k_operands(k_stage[1]);
+    }
+    // Rows travel two iterations in registers (K(m+5) and V(m+2) are requested in
+    // iteration m and written to LDS in iteration m+2), and their page ids are
+    // looked up two iterations before that.  Even and odd iterations own a
+    // register set each.  K has three LDS stages, so that the operands of S(m+2)
+    // can be read while iteration m still multiplies.
+    const int v_lane_off = (4 * h + (c >> 2)) * kPVPitch + (g & 1) * 32 + (c & 3) * 8;
+    int k_store = 0, k_next = 2;   // m % 3 and (m + 2) % 3
+    auto iteration = [&](int m, RowSet &rows) {
         __syncthreads();
-        store_rows(stage[cur ^ 1], regs);
-        load_rows(t + 2 * kBlock, regs);
-        if (t < w_end) compute_block(t, stage[cur]);
+        store_rows(k_stage[k_store], kKPitch, rows.k);
+        store_rows(v_stage[m & 1], kPVPitch, rows.v);
+        load_rows(m + 5, 0, rows.k_pg, rows.k);
+        load_rows(m + 2, half_bytes, rows.v_pg, rows.v);
+        lookup_pages(m + 7, rows.k_pg);
+        lookup_pages(m + 4, rows.v_pg);
+        const char *k_ahead = k_stage[k_next];
+        k_store = k_store == 2 ? 0 : k_store + 1;
+        k_next = k_next == 2 ? 0 : k_next + 1;
+        if (!(w_end > 0 && (m - 1) * kBlock < w_end)) return;
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+            // rare: raise the maximum and bring what was computed under the old
+            // one (accumulators, row sum, the pending P(m-1)) to the new scale
+            const float m_new = fmaxf(m_run, m_blk);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) acc[dt] *= alpha;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    float lo, hi;
+                    E::unpack2(pb[ks][w], lo, hi);
+                    pb[ks][w] = E::pack2(lo * alpha, hi * alpha);
+                }
+        }
+        // The rest of the iteration is two straight-line halves, each an MFMA
+        // strand with independent vector work in its shadow:
+        //   S(m+1) = K(m+1).Q^T     |  P(m) = exp2(S(m) * scale - max), packed; row sum;
+        //                           |  V(m-1) operands from LDS
+        //   O += P(m-1).V(m-1)      |  maximum of S(m+1); K(m+2) operands from LDS
+        // with the masking of S(m+1), where needed, between them.  A masked score
+        // is kNegBig and the maximum never drops below its start value, so masked
+        // probabilities come out as exp2(-huge) = 0 without a select.
+        float s_cur[16];
+        u32x4 pb_prev[2];
+        pb_prev[0] = pb[0];
+        pb_prev[1] = pb[1];
+#pragma unroll
+        for (int v = 0; v < 16; v++) s_cur[v] = x[v];
+        // V operand: the transposing read hands each block of 16 lanes four tokens
+        // of 16 consecutive dims, lane i of the block supplying the address of dims
+        // 4*(i%4) .. +3 of the block's token i/4
+        const char *v_rows = v_stage[(m - 1) & 1] + v_lane_off;
+        u32x4 va[4][2];
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const char *vp = v_rows + ks * 16 * kPVPitch + dt * 64;
+                const u32x2 a_lo = read_transposed(vp);
+                const u32x2 a_hi = read_transposed(vp + 8 * kPVPitch);
+                va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
+            }
+        scores();
+        {
+            float p[16], p_sum = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[v], scale_log2, -m_run));
+                p_sum += p[v];
+            }
+            l_run += p_sum;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+                pb[ks] = u32x4{E::pack2(p[8 * ks], p[8 * ks + 1]), E::pack2(p[8 * ks + 2], p[8 * ks + 3]),
+                               E::pack2(p[8 * ks + 4], p[8 * ks + 5]), E::pack2(p[8 * ks + 6], p[8 * ks + 7])};
+        }
+        // keeps P(m) in this half (it is only consumed by the next iteration)
+        asm volatile("" ::"v"(pb[0]), "v"(pb[1]), "v"(l_run));
+        if ((m + 2) * kBlock > w_mask_from) mask_scores(m + 1);   // wave-uniform
+
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) acc[dt] = E::mfma_32x32(va[dt][ks], pb_prev[ks], acc[dt]);
+        block_max();
+        read_k_operands(k_ahead);   // K(m+2), for the next iteration
+        asm volatile("" ::"v"(m_blk));
+    };
+    for (int m = 0; m <= n_blocks; m += 2) {
+        iteration(m, even);
+        iteration(m + 1, odd);
     }
 
-#pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        float l = l_run[ct];
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
-        const int qrow = wq0 + ct * pos_per_ct + c_pos;
-        if (!(c_used && qrow < n_b)) continue;
+    float l_other = l_run;
+    swap_halves32(l_run, l_other);
+    const float l = l_run + l_other;
+    if (live) {
         const float inv = l > 0.f ? 1.f / l : 0.f;
         uint16_t *o = out + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim +
-                      4 * g;
+                      4 * h;
 #pragma unroll
-        for (int dt = 0; dt < 8; dt++) {
-            u32x2 w = {E::pack2(acc[ct][dt][0] * inv, acc[ct][dt][1] * inv),
-                       E::pack2(acc[ct][dt][2] * inv, acc[ct][dt][3] * inv)};
-            *reinterpret_cast<u32x2 *>(o + dt * 16) = w;
-        }
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                u32x2 w = {E::pack2(acc[dt][4 * i] * inv, acc[dt][4 * i + 1] * inv),
+                           E::pack2(acc[dt][4 * i + 2] * inv, acc[dt][4 * i + 3] * inv)};
+                *reinterpret_cast<u32x2 *>(o + dt * 32 + 8 * i) = w;
+            }
     }
 }
 
@@ -348,7 +463,7 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
 static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads)
 {
     const int group = n_qo_heads / n_kv_heads;
-    return group <= 16 ? kPrefillWaves * kColTiles * (16 / group) : 1;
+    return group <= kWaveCols ? kPrefillWaves * (kWaveCols / group) : 1;
 }
 
 }  // namespace dskv
@@ -420,7 +535,7 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     hipStream_t s = (hipStream_t)stream;
     // the MFMA kernel takes maxima before scaling: it needs a positive, sane scale
     const bool mfma = (dtype == DSKV_BF16 || dtype == DSKV_F16) && head_dim == kHeadDim &&
-                      n_qo_heads / n_kv_heads <= 16 && scale_log2 > 1e-6f && scale_log2 < 1e6f;
+                      n_qo_heads / n_kv_heads <= kWaveCols && scale_log2 > 1e-6f && scale_log2 < 1e6f;
     if (mfma) {
         DSKV_REQUIRE(tile_info_dev && n_tiles > 0, "prefill_attn: missing tile list");
         DSKV_REQUIRE(((uintptr_t)out | (uintptr_t)q | (uintptr_t)pages_layer) % 16 == 0,

@@ -231,6 +231,9 @@ PREFILL_CASES = [
     ("mha", [100, 20], [30, 20], 16, 8, 8, 128, "bf16"),
     ("f32", [60, 20], [30, 20], 16, 8, 2, 128, "f32"),
     ("empty_chunk", [60, 20, 40], [30, 0, 5], 16, 32, 8, 128, "bf16"),
+    ("page2", [130, 45, 7], [64, 45, 2], 2, 32, 8, 128, "bf16"),
+    ("page4_group16", [200, 33], [70, 33], 4, 32, 2, 128, "f16"),
+    ("long_tile", [900], [300], 16, 32, 8, 128, "bf16"),
 ]
 
 
