@@ -149,7 +149,8 @@ def test_prefill_plan_tiles_cover_all_query_rows():
                 continue
             if rows is None:
                 rows = starts[1] - starts[0] if len(starts) > 1 else nb
-                assert rows % max(16 // group, 1) == 0 if group <= 16 else rows == 1
+                # a tile is a whole number of waves, each 32 // group query rows
+                assert rows % max(32 // group, 1) == 0 if group <= 32 else rows == 1
             assert starts == list(range(0, nb, rows))
     n = ctypes.c_int32()
     assert lib.dskv_prefill_plan(qo.ctypes.data, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2
