@@ -28,6 +28,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_BF16_TFLOPS = 2500.0
 
 
 def parse_args():
@@ -40,6 +41,7 @@ def parse_args():
     ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill section")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -211,6 +213,76 @@ def swap_section(seed: int):
             "decode_steps_during_swap": steps}
 
 
+def prefill_section(seed: int):
+    """Baseline configuration 4 (Llama-3-8B stage): 16 sequences each append a 512-token chunk
+    at a start offset U[0,15] inside a partially filled page and attend over a prior context
+    U[0,8192].  Timed per layer on the launch stream: the chunk append and the paged prefill
+    attention (4 layers of the stage's 16 are allocated; the layers are identical work)."""
+    import numpy as np
+    import torch
+
+    from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.model.context.flash import FlashPrefillCtx
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper, append_paged_kv_cache
+    from deserve_amd.synthetic import fill_normal, scatter_pool_order
+    from deserve_amd.task import SamplingParams, TaskData
+
+    dev = torch.device("cuda")
+    L, P, Hq, Hkv, D, B, n = 4, 16, 32, 8, 128, 16, 512
+    rng = np.random.default_rng(seed + 40)
+    prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
+    pool = GpuPagePool(L, int((-(-(prior + n) // P)).sum()) + 8, P, dev, torch.bfloat16)
+    fill_normal(pool.pages, seed + 41)
+    scatter_pool_order(pool, seed + 42)
+    rows = PageTableAllocator(B, 8192 + 1024, P, dev)
+    tasks = [TaskData(f"p{b}", int(prior[b]), 1, n, int(prior[b]) + n, SamplingParams()) for b in range(B)]
+    caches = [PagedKVCache.empty(rows, pool) for _ in range(B)]
+    gen = torch.Generator(device="cuda").manual_seed(seed + 43)
+    q = torch.randn((L, B * n, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
+    k = torch.randn((L, B * n, Hkv, D), device=dev, generator=gen).to(torch.bfloat16)
+    v = torch.randn((L, B * n, Hkv, D), device=dev, generator=gen).to(torch.bfloat16)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device=dev))
+    c = FlashPrefillCtx.init_paged_prefill_ctx(tasks, caches, w)
+    w.begin_forward(qo_indptr=c.indptr, paged_kv_indptr=c.kv_page_indptr,
+                    paged_kv_indices=c.kv_page_indices, paged_kv_last_page_len=c.kv_last_page_lens,
+                    num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
+                    qo_indptr_host=c.host["indptr"])
+    flops = 4 * Hq * D * sum(n * int(p) + n * (n + 1) // 2 for p in prior)
+
+    def median_us(fn, reps=5):
+        evs = []
+        for _ in range(reps):
+            for layer in range(L):
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                fn(layer)
+                e.record()
+                evs.append((s, e))
+        torch.cuda.synchronize()
+        ts = sorted(s.elapsed_time(e) for s, e in evs)
+        return ts[len(ts) // 2] * 1e3
+
+    def append(layer):
+        append_paged_kv_cache(k[layer], v[layer], c.indptr, pool.pages[layer], c.kv_page_indices,
+                              c.kv_page_indptr, c.kv_last_page_lens)
+
+    append_us = median_us(append)
+    attn_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
+    w.end_forward()
+    append_bytes = 2 * B * n * 2 * Hkv * D * 2
+    return {"workload": "BASELINE.json configs[3]: bf16, GQA 32q/8kv, page 16, 16 sequences x 512-token "
+                        "chunk appended at offsets U[0,15], attention over prior U[0,8192]; per layer",
+            "chunk_tokens": B * n, "kv_tokens": int((prior + n).sum()),
+            "append_us_per_layer": round(append_us, 1),
+            "append_GBps": round(append_bytes / append_us / 1e3, 1),
+            "attention_us_per_layer": round(attn_us, 1),
+            "attention_TFLOPs": round(flops / attn_us / 1e6, 1),
+            "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
+            "flops_per_layer": flops}
+
+
 def main() -> int:
     a = parse_args()
     if a.gpus != 1:
@@ -337,10 +409,13 @@ def main() -> int:
     if not a.no_cpu_baseline:
         meta = {n: last_ctx.host[n].numpy() for n in ("kv_page_indices", "kv_page_indptr", "kv_last_page_lens")}
         out["cpu_baseline"] = cpu_baseline(wl, meta, sample_requests=16)
+    del wl, last_ctx
+    torch.cuda.empty_cache()
     if not a.no_swap:
-        del wl, last_ctx
-        torch.cuda.empty_cache()
         out["swap"] = swap_section(a.seed)
+        torch.cuda.empty_cache()
+    if not a.no_prefill:
+        out["prefill"] = prefill_section(a.seed)
     print(json.dumps(out))
     return 0
 
