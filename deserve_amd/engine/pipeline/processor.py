@@ -37,6 +37,36 @@ class StepRequest:
     reload_task_ids: List[str] = field(default_factory=list)
     init_tasks: Dict[str, Tuple[int, SamplingParams]] = field(default_factory=dict)
 
+    @staticmethod
+    def empty(group_id: int, dtype: torch.dtype, device=None) -> "StepRequest":
+        from deserve_amd.task import main_device
+        return StepRequest(group_id, torch.empty((0,), dtype=dtype, device=device or main_device))
+
+    def is_empty(self) -> bool:
+        return (self.xs.numel() == 0 and not self.exec_task_ids and not self.exec_seqlens
+                and not self.cancel_task_ids and not self.offload_task_ids
+                and not self.reload_task_ids and not self.init_tasks)
+
+    def append_exec(self, task_id: str, x: torch.Tensor, init_info=None) -> None:
+        """Adds a task's tokens to the batch (request.py:172-188); init_info =
+        (initial_seqlen, SamplingParams) for a task seen for the first time."""
+        assert x.numel() > 0
+        self.exec_task_ids.append(task_id)
+        self.exec_seqlens.append(x.shape[0])
+        self.xs = x if self.xs.numel() == 0 else torch.cat([self.xs, x], dim=0)
+        if init_info is not None:
+            self.init_tasks[task_id] = init_info
+
+    def get_bsz(self) -> int:
+        return len(self.exec_task_ids)
+
+    def refresh(self) -> None:
+        """A request that comes round again carries only decodes (request.py:193-197)."""
+        self.offload_task_ids = []
+        self.reload_task_ids = []
+        self.exec_seqlens = [1] * len(self.exec_task_ids)
+        self.init_tasks = {}
+
 
 class PipelineProcessor:
     def __init__(self, num_rounds: int, num_pages_main: int, num_pages_swap: int, page_size: int,
@@ -62,6 +92,7 @@ class PipelineProcessor:
         self.current_microbatch_id = 0
         self.ignore_eos = ignore_eos
         self.last_result: BatchResult = None   # type: ignore[assignment]
+        self.last_exec = ([], [], None)        # what the last step ran: task ids, seqlens, inputs
 
     def synchronize(self) -> None:
         pool = self.virtual_page_pool
@@ -94,6 +125,7 @@ class PipelineProcessor:
                   [self.offloaded_kvcaches.pop(tid) for tid in request.reload_task_ids])
         mb.kvcache_manager.synchronize()
 
+        self.last_exec = (list(request.exec_task_ids), list(request.exec_seqlens), request.xs)
         if request.exec_task_ids:
             mb.join(list(request.init_tasks.keys()))
             result = mb.step(request.exec_task_ids, request.xs, prev_mb, next_mb)

@@ -47,3 +47,18 @@ class KVStage:
             outs.append(self.core.paged_forward(q[layer], k[layer], v[layer], ctx))
             ctx.layer_id += 1
         return torch.stack(outs)
+
+
+class PackedKVStage(KVStage):
+    """KVStage for callers that carry one tensor per token, as the scheduler's
+    queues do: xs is (nnz, L, Hq + 2*Hkv, D) with each token's q, k and v heads of
+    every layer side by side."""
+
+    def forward(self, xs: torch.Tensor, ctx: FlashForwardCtx) -> torch.Tensor:   # type: ignore[override]
+        hq = self.model_args.n_heads
+        hkv = hq if self.model_args.n_kv_heads is None else self.model_args.n_kv_heads
+        by_layer = xs.permute(1, 0, 2, 3)
+        q = by_layer[:, :, :hq].contiguous()
+        k = by_layer[:, :, hq:hq + hkv].contiguous()
+        v = by_layer[:, :, hq + hkv:].contiguous()
+        return super().forward((q, k, v), ctx)

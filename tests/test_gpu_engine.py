@@ -140,3 +140,90 @@ def test_offload_reload_and_cancel_through_the_stage_driver():
     run(0, ["a", "b"], [1, 1], cancel_task_ids=["c"])
     assert "c" not in proc.microbatches[0].ongoing_paged_kvcaches
     assert proc.cpu_chunk_pool.available_ids[-1] == [0]              # the chunk was returned
+
+
+@pytest.mark.parametrize("policy", ["decode_first", "prefill_first", "vanilla"])
+def test_scheduler_policies_under_page_pressure(policy):
+    """Prompts arrive faster than the pool can hold them: the join stage batches, the
+    swap stage evicts to pinned memory and reloads when cancelled tasks free pages.
+    Whatever the policy decides, every executed token must attend to exactly its own
+    request's history."""
+    from deserve_amd.engine.pipeline.processor import StepRequest
+    from deserve_amd.engine.pipeline.scheduler import PipelineScheduler
+    from deserve_amd.stage import PackedKVStage, StageArgs
+    from deserve_amd.task import SamplingParams
+
+    print("[case] scheduler", policy, flush=True)
+    rng = np.random.default_rng({"decode_first": 1, "prefill_first": 2, "vanilla": 3}[policy])
+    stage = PackedKVStage(StageArgs(n_heads=HQ, n_kv_heads=HKV, dim=HQ * D, page_size=P, n_layers=L),
+                          use_rope=False)
+    sched = PipelineScheduler(num_rounds=2, num_pages_main=10, num_pages_swap=6, page_size=P,
+                              batch_size=8, layer_storage=stage, num_layers=L, buddy_height=7,
+                              main_dtype=torch.bfloat16, max_context_len=512,
+                              decode_first_aggregate=policy == "decode_first",
+                              prefill_first_aggregate=policy == "prefill_first",
+                              max_aggregated_tokens=48)
+    sched.virtual_page_pool.pages.view(torch.int16).fill_(0x7FC0)
+    shadow = Shadow()
+    width = HQ + 2 * HKV
+
+    def rows(n):
+        bits = _bf(rng.standard_normal((n, L, width, D)).astype(np.float32))
+        return _to_dev(bits)
+
+    def bits_of(x):
+        return x.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    # prompts end just short of a page boundary and decode across one or two: the running
+    # batch outgrows the 16 pages it was admitted into
+    prompt_len = {f"t{i}": n for i, n in enumerate([30, 46, 62, 31, 47, 29, 45])}
+    arrivals = {0: ["t0", "t1"], 1: ["t2"], 2: ["t3", "t4"], 5: ["t5"], 9: ["t6"]}
+    decode_budget = {t: int(n) for t, n in zip(prompt_len, rng.integers(18, 30, size=7))}
+    decoded = {t: 0 for t in prompt_len}
+    finished, offloads, reloads = set(), 0, 0
+    requests = [StepRequest.empty(m, torch.bfloat16, DEV) for m in range(2)]
+    for step in range(400):
+        for t in arrivals.get(step, []):
+            sched.process_init(t, rows(prompt_len[t]), SamplingParams())
+        m = step % 2
+        req = requests[m]
+        sched.synchronize()
+        req = sched.process_step(req)
+        torch.cuda.synchronize()
+        offloads += len(req.offload_task_ids)
+        reloads += len(req.reload_task_ids)
+        ids, seqlens, xs = sched.last_exec
+        if ids:
+            got = sched.last_result.all_xs.float().cpu().numpy().reshape(L, sum(seqlens), HQ, D)
+            assert np.isfinite(got).all(), (step, "a stale or foreign page was read")
+            xb = bits_of(xs)
+            pos = 0
+            for t, n in zip(ids, seqlens):
+                chunk = xb[pos: pos + n]
+                for layer in range(L):
+                    want = shadow.expect(t, layer, chunk[:, layer, :HQ], chunk[:, layer, HQ:HQ + HKV],
+                                         chunk[:, layer, HQ + HKV:])
+                    assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
+                pos += n
+        # a task that has produced its budget of tokens is cancelled on its next round;
+        # one that is still prefilling has no next input yet and drops out of the batch
+        keep, keep_rows, cancel = [], [], []
+        for i, t in enumerate(req.exec_task_ids):
+            d = sched.task_manager.get(t)
+            if d.seqlen == 0:
+                continue
+            decoded[t] += 1
+            if decoded[t] >= decode_budget[t]:
+                cancel.append(t)
+                finished.add(t)
+            else:
+                keep.append(t)
+        req.exec_task_ids = keep
+        req.xs = rows(len(keep)) if keep else torch.empty((0,), dtype=torch.bfloat16, device=DEV)
+        req.cancel_task_ids = cancel
+        requests[m] = req
+        if len(finished) == len(prompt_len):
+            break
+    sched.synchronize()
+    assert finished == set(prompt_len), (finished, decoded)
+    assert offloads > 0 and reloads > 0, (offloads, reloads)
