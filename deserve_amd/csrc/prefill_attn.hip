@@ -58,8 +58,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     int n_kv_heads, int page_shift, float scale_log2, int causal)
 {
     typedef Elt<DT> E;
-    __shared__ __align__(16) char k_stage[3][kBlock * kKPitch];
-    __shared__ __align__(16) char v_stage[2][kBlock * kPVPitch];
+    __shared__ __align__(16) char k_stage[2][kBlock * kKPitch];
+    __shared__ __align__(16) char v_stage[4][kBlock * kPVPitch];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -155,28 +155,34 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
             pg[i] = __builtin_amdgcn_raw_buffer_load_b32(page_table, (tok0 >> page_shift) * 4 + lane * 0, 0, 0);
         }
     };
-    auto load_rows = [&](int blk, int half_off, const int(&pg)[kRowGroups], u32x4(&rows)[kRowGroups]) {
+    auto load_rows = [&](int blk, const int(&pg)[kRowGroups], u32x4(&k_rows)[kRowGroups],
+                         u32x4(&v_rows)[kRowGroups]) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
             const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
             if (kRowsSharePage) {
-                // one page holds the 4 rows: a descriptor that ends after the last
-                // valid row makes the bounds check free and keeps offsets constant
+                // one page holds the 4 rows: descriptors that end after the last
+                // valid row make the bounds check free and keep offsets constant
                 const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
                 const long page = __builtin_amdgcn_readfirstlane(pg[i]);
-                char *first_row = const_cast<char *>(pages) + page * page_bytes + half_off +
+                char *first_row = const_cast<char *>(pages) + page * page_bytes +
                                   (long)(tok0 & page_mask) * row_bytes;
-                __amdgpu_buffer_rsrc_t desc = __builtin_amdgcn_make_buffer_rsrc(
+                __amdgpu_buffer_rsrc_t k_desc = __builtin_amdgcn_make_buffer_rsrc(
                     first_row, 0, valid * row_bytes, kBufferFlags);
-                rows[i] = __builtin_amdgcn_raw_buffer_load_b128(desc, lane_off, 0, kLoadCached);
+                __amdgpu_buffer_rsrc_t v_desc = __builtin_amdgcn_make_buffer_rsrc(
+                    first_row + half_bytes, 0, valid * row_bytes, kBufferFlags);
+                k_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(k_desc, lane_off, 0, kLoadCached);
+                v_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(v_desc, lane_off, 0, kLoadCached);
             } else {
                 const int tok = tok0 + g;
                 const int tc = min(tok, t_end - 1);
-                const char *p = pages + page_ids[tc >> page_shift] * page_bytes + half_off +
+                const char *p = pages + page_ids[tc >> page_shift] * page_bytes +
                                 (long)(tc & page_mask) * row_bytes + (lane_off - g * row_bytes);
                 const u32x4 z = {0, 0, 0, 0};
-                const u32x4 got = *reinterpret_cast<const u32x4 *>(p);
-                rows[i] = tok < t_end ? got : z;
+                const u32x4 got_k = *reinterpret_cast<const u32x4 *>(p);
+                const u32x4 got_v = *reinterpret_cast<const u32x4 *>(p + half_bytes);
+                k_rows[i] = tok < t_end ? got_k : z;
+                v_rows[i] = tok < t_end ? got_v : z;
             }
         }
     };
@@ -231,72 +237,60 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         raise = m_blk > m_run + kRescaleSlack;
     };
 
-    // The K rows run two blocks ahead of the V rows: iteration m of the main loop
-    // multiplies P(m-1) into V(m-1), turns S(m) into P(m) and computes S(m+1), so
-    // that every MFMA of the iteration is independent of its exponentials and the
-    // matrix and vector pipelines of a wave overlap.  Per iteration one barrier:
-    // past it K(m+2) and V(m-1) are complete, and the stages that held K(m) and
-    // V(m-2) are free for K(m+3) and V(m).  Every wave runs every iteration (idle
-    // ones only move rows), so the barriers match.
+    // Iteration m of the main loop multiplies P(m-1) into V(m-1), turns S(m) into
+    // P(m) and computes S(m+1), so that every MFMA of the iteration is independent
+    // of its exponentials and the matrix and vector pipelines of a wave overlap.
+    // The rows of block m+4 are requested in iteration m (their page id was looked
+    // up in iteration m-2) and written to LDS in iteration m+2: one iteration is
+    // shorter than a trip to memory.  K has two LDS stages and V four (V(j) is
+    // read three iterations after it is stored).  Per iteration one barrier: past
+    // it K(m+1) and V(m-1) are complete and the stages of K(m) and V(m-2) are free.
+    // Every wave runs every iteration (idle ones only move rows), so the barriers
+    // match.  The loop is unrolled by four so that all stage indices are static.
     struct RowSet {
-        u32x4 k[kRowGroups], v[kRowGroups];       // rows on their way to LDS
-        int k_pg[kRowGroups], v_pg[kRowGroups];   // page ids of the rows requested next
+        u32x4 k[kRowGroups], v[kRowGroups];   // rows on their way to LDS
+        int pg[kRowGroups];                   // page ids of the rows requested next
     };
     RowSet even, odd;
     {
         int pg[kRowGroups];
-        u32x4 first[3][kRowGroups];
+        u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
 #pragma unroll
-        for (int blk = 0; blk < 3; blk++) {
+        for (int blk = 0; blk < 2; blk++) {
             lookup_pages(blk, pg);
-            load_rows(blk, 0, pg, first[blk]);
+            load_rows(blk, pg, first_k[blk], first_v[blk]);
         }
+        lookup_pages(2, even.pg);
+        lookup_pages(3, odd.pg);
         const u32x4 z = {0, 0, 0, 0};
         u32x4 zero[kRowGroups];
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) zero[i] = z;
-        store_rows(v_stage[1], kPVPitch, zero);   // V(-1): multiplied by P(-1) = 0, must be finite
+        store_rows(v_stage[3], kPVPitch, zero);   // V(-1): multiplied by P(-1) = 0, must be finite
 #pragma unroll
-        for (int blk = 0; blk < 3; blk++) store_rows(k_stage[blk], kKPitch, first[blk]);
+        for (int blk = 0; blk < 2; blk++) {
+            store_rows(k_stage[blk], kKPitch, first_k[blk]);
+            store_rows(v_stage[blk], kPVPitch, first_v[blk]);
+        }
     }
-    lookup_pages(3, even.k_pg);
-    lookup_pages(4, odd.k_pg);
-    lookup_pages(0, even.v_pg);
-    lookup_pages(1, odd.v_pg);
-    load_rows(3, 0, even.k_pg, even.k);
-    load_rows(4, 0, odd.k_pg, odd.k);
-    load_rows(0, half_bytes, even.v_pg, even.v);
-    load_rows(1, half_bytes, odd.v_pg, odd.v);
-    lookup_pages(5, even.k_pg);
-    lookup_pages(6, odd.k_pg);
-    lookup_pages(2, even.v_pg);
-    lookup_pages(3, odd.v_pg);
+    load_rows(2, even.pg, even.k, even.v);
+    load_rows(3, odd.pg, odd.k, odd.v);
+    lookup_pages(4, even.pg);
+    lookup_pages(5, odd.pg);
     __syncthreads();
     if (w_end > 0) {
         read_k_operands(k_stage[0]);
         scores();
         if (kBlock > w_mask_from) mask_scores(0);
         block_max();
-        read_k_operands(k_stage[1]);
     }
-    // Rows travel two iterations in registers (K(m+5) and V(m+2) are requested in
-    // iteration m and written to LDS in iteration m+2), and their page ids are
-    // looked up two iterations before that.  Even and odd iterations own a
-    // register set each.  K has three LDS stages, so that the operands of S(m+2)
-    // can be read while iteration m still multiplies.
     const int v_lane_off = (4 * h + (c >> 2)) * kPVPitch + (g & 1) * 32 + (c & 3) * 8;
-    int k_store = 0, k_next = 2;   // m % 3 and (m + 2) % 3
-    auto iteration = [&](int m, RowSet &rows) {
+    auto iteration = [&](int m, int phase, RowSet &rows) {   // phase = m % 4, a literal at each call
         __syncthreads();
-        store_rows(k_stage[k_store], kKPitch, rows.k);
-        store_rows(v_stage[m & 1], kPVPitch, rows.v);
-        load_rows(m + 5, 0, rows.k_pg, rows.k);
-        load_rows(m + 2, half_bytes, rows.v_pg, rows.v);
-        lookup_pages(m + 7, rows.k_pg);
-        lookup_pages(m + 4, rows.v_pg);
-        const char *k_ahead = k_stage[k_next];
-        k_store = k_store == 2 ? 0 : k_store + 1;
-        k_next = k_next == 2 ? 0 : k_next + 1;
+        store_rows(k_stage[phase & 1], kKPitch, rows.k);              // K(m+2)
+        store_rows(v_stage[(phase + 2) & 3], kPVPitch, rows.v);       // V(m+2)
+        load_rows(m + 4, rows.pg, rows.k, rows.v);
+        lookup_pages(m + 6, rows.pg);
         if (!(w_end > 0 && (m - 1) * kBlock < w_end)) return;
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
             // rare: raise the maximum and bring what was computed under the old
@@ -320,7 +314,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         // strand with independent vector work in its shadow:
         //   S(m+1) = K(m+1).Q^T     |  P(m) = exp2(S(m) * scale - max), packed; row sum;
         //                           |  V(m-1) operands from LDS
-        //   O += P(m-1).V(m-1)      |  maximum of S(m+1); K(m+2) operands from LDS
+        //   O += P(m-1).V(m-1)      |  maximum of S(m+1)
         // with the masking of S(m+1), where needed, between them.  A masked score
         // is kNegBig and the maximum never drops below its start value, so masked
         // probabilities come out as exp2(-huge) = 0 without a select.
@@ -333,7 +327,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         // V operand: the transposing read hands each block of 16 lanes four tokens
         // of 16 consecutive dims, lane i of the block supplying the address of dims
         // 4*(i%4) .. +3 of the block's token i/4
-        const char *v_rows = v_stage[(m - 1) & 1] + v_lane_off;
+        read_k_operands(k_stage[(phase + 1) & 1]);                       // K(m+1)
+        const char *v_rows = v_stage[(phase + 3) & 3] + v_lane_off;        // V(m-1)
         u32x4 va[4][2];
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
@@ -367,12 +362,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) acc[dt] = E::mfma_32x32(va[dt][ks], pb_prev[ks], acc[dt]);
         block_max();
-        read_k_operands(k_ahead);   // K(m+2), for the next iteration
         asm volatile("" ::"v"(m_blk));
     };
-    for (int m = 0; m <= n_blocks; m += 2) {
-        iteration(m, even);
-        iteration(m + 1, odd);
+    for (int m = 0; m <= n_blocks; m += 4) {
+        iteration(m, 0, even);
+        iteration(m + 1, 1, odd);
+        iteration(m + 2, 2, even);
+        iteration(m + 3, 3, odd);
     }
 
     float l_other = l_run;
