@@ -287,7 +287,8 @@ def main() -> int:
     a = parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {a.gpus} is not supported in this build "
-              "(the path has no cross-GPU exchange; see DESIGN.md on sharding)", file=sys.stderr)
+              "(the path has no cross-GPU exchange: it shards by layers, kv heads or sequences "
+              "with one independent copy of this work per GPU)", file=sys.stderr)
         return 2
     import numpy as np
     import torch
