@@ -73,8 +73,11 @@ struct LoadCursor {
     long page;                 // pool page of tile t, fetched one tile ahead of its use
 };
 
+#ifndef DSKV_DECODE_MIN_WAVES
+#define DSKV_DECODE_MIN_WAVES 1
+#endif
 template <int DT, bool kPageCoversTile>
-__global__ __launch_bounds__(64 * kMaxWaves) void decode_attn_mfma_kernel(
+__global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_attn_mfma_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ q, const char *__restrict__ pages,
     const int32_t *__restrict__ kv_indices, const Item *__restrict__ items,
     const int32_t *__restrict__ wg_ptr, float *__restrict__ part_o, float *__restrict__ part_ml,
