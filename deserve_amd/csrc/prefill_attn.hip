@@ -34,7 +34,11 @@ namespace dskv {
 #define DSKV_PREFILL_VPITCH 320
 #endif
 constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
-constexpr int kWaveCols = 32;                       // columns per wave (one MFMA tile)
+#ifndef DSKV_PREFILL_COLTILES
+#define DSKV_PREFILL_COLTILES 1
+#endif
+constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
+constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
 constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
 constexpr int kKPitch = DSKV_PREFILL_KPITCH;        // bytes per K row in LDS (256 + pad)
 constexpr int kPVPitch = DSKV_PREFILL_VPITCH;       // bytes per V row in LDS (256 + pad)
@@ -84,22 +88,26 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     const long page_bytes = 2L * half_bytes;
     const int page_mask = (1 << page_shift) - 1;
 
-    // column r: query row wq0 + r/group, head r%group
+    // column r of column tile ct: query row wq0 + (32 ct + r)/group, head (32 ct + r)%group
     const int wq0 = q0 + wave * pos_per_wave;
-    const int c_pos = r / group;
-    const int c_head = r - c_pos * group;
-    const int qrow = wq0 + c_pos;
-    const bool live = c_pos < pos_per_wave && qrow < n_b;
-    int limit = causal ? kv_len - n_b + qrow + 1 : kv_len;   // kv tokens this column may see
-    limit = live ? min(max(limit, 0), kv_len) : 0;
-    u32x4 qreg[8];     // dims 16*ks + 8h .. +7 of the column's query
-    {
+    int qrow[kColTiles], c_head[kColTiles], limit[kColTiles];   // limit: kv tokens the column may see
+    bool live[kColTiles];
+    u32x4 qreg[kColTiles][8];     // dims 16*ks + 8h .. +7 of the column's query
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ct++) {
+        const int col = 32 * ct + r;
+        const int c_pos = col / group;
+        c_head[ct] = col - c_pos * group;
+        qrow[ct] = wq0 + c_pos;
+        live[ct] = c_pos < pos_per_wave && qrow[ct] < n_b;
+        const int lim = causal ? kv_len - n_b + qrow[ct] + 1 : kv_len;
+        limit[ct] = live[ct] ? min(max(lim, 0), kv_len) : 0;
         const uint16_t *qrow_p =
-            q + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim + h * 8;
+            q + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim + h * 8;
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             u32x4 z = {0, 0, 0, 0};
-            qreg[ks] = live ? *reinterpret_cast<const u32x4 *>(qrow_p + ks * 16) : z;
+            qreg[ct][ks] = live[ct] ? *reinterpret_cast<const u32x4 *>(qrow_p + ks * 16) : z;
         }
     }
     // Token ranges from scalars only: they steer loops, barriers and page lookups
@@ -116,20 +124,27 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     const int n_blocks = (t_end + kBlock - 1) / kBlock;
     // Start value of the running maximum: far below any scaled score, far above a
     // scaled masked score (kNegBig * scale_log2).
-    float m_run = 0.5f * kNegBig * scale_log2, l_run = 0.f;
-    f32x16 acc[4];     // O^T: dims 32*dt + 8i + 4h + j of column r in acc[dt][4i + j]
-    u32x4 pb[2];       // packed probabilities of the previous block, per k-step
+    float m_run[kColTiles], l_run[kColTiles];
+    f32x16 acc[kColTiles][4];     // O^T: dims 32*dt + 8i + 4h + j of column r in acc[ct][dt][4i + j]
+    u32x4 pb[kColTiles][2];       // packed probabilities of the previous block, per k-step
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+    for (int ct = 0; ct < kColTiles; ct++) {
+        m_run[ct] = 0.5f * kNegBig * scale_log2;
+        l_run[ct] = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[dt][v] = 0.f;
-    pb[0] = pb[1] = u32x4{0, 0, 0, 0};
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[ct][dt][v] = 0.f;
+        pb[ct][0] = pb[ct][1] = u32x4{0, 0, 0, 0};
+    }
 
     // No kv token visible to any row of the tile: the output rows are zero.
     // (Uniform over the workgroup, and before the first barrier.)
     if (t_end == 0) {
-        if (live) {
-            uint16_t *o = out + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim +
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ct++) {
+            if (!live[ct]) continue;
+            uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
                           4 * h;
 #pragma unroll
             for (int i = 0; i < 16; i++) *reinterpret_cast<u32x2 *>(o + 8 * i) = u32x2{0, 0};
@@ -198,7 +213,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
     // x[4i + j].  Registers 8s .. 8s+7, packed, are the B operand of the P.V MFMA
     // for k-step s, which thereby fixes the tokens of that step's k slots:
     // 16s + 4h + j in slots j, 16s + 8 + 4h + j in slots 4 + j.
-    float x[16];
+    float x[kColTiles][16];
     u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
     auto read_k_operands = [&](const char *kst) {
         const char *k_rows = kst + r * kKPitch + h * 16;
@@ -206,35 +221,48 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 32);
     };
     auto scores = [&]() {
-        f32x16 s;
+        f32x16 s[kColTiles];
 #pragma unroll
-        for (int v = 0; v < 16; v++) s[v] = 0.f;
+        for (int ct = 0; ct < kColTiles; ct++)
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) s = E::mfma_32x32(ka[ks], qreg[ks], s);
+            for (int v = 0; v < 16; v++) s[ct][v] = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) x[v] = s[v];
+        for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+            for (int ct = 0; ct < kColTiles; ct++) s[ct] = E::mfma_32x32(ka[ks], qreg[ct][ks], s[ct]);
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ct++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) x[ct][v] = s[ct][v];
     };
     // Masks block blk's scores (needed from w_mask_from on).
     auto mask_scores = [&](int blk) {
         const int t = blk * kBlock;
 #pragma unroll
-        for (int v = 0; v < 16; v++)
-            if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit) x[v] = kNegBig;
+        for (int ct = 0; ct < kColTiles; ct++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit[ct]) x[ct][v] = kNegBig;
     };
     // Column maximum of the block in x, and whether the running maximum has to be
     // raised before the block's exponentials.
-    float m_blk = 0.f;
+    float m_blk[kColTiles];
     bool raise = false;
     auto block_max = [&]() {
-        // scale_log2 > 0: the maximum can be taken before scaling
-        float m = fmaxf(fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])),
-                              fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7]))),
-                        fmaxf(fmaxf(fmaxf(x[8], x[9]), fmaxf(x[10], x[11])),
-                              fmaxf(fmaxf(x[12], x[13]), fmaxf(x[14], x[15]))));
-        float other = m;
-        swap_halves32(m, other);
-        m_blk = fmaxf(m, other) * scale_log2;
-        raise = m_blk > m_run + kRescaleSlack;
+        raise = false;
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ct++) {
+            const float *xc = x[ct];
+            // scale_log2 > 0: the maximum can be taken before scaling
+            float m = fmaxf(fmaxf(fmaxf(fmaxf(xc[0], xc[1]), fmaxf(xc[2], xc[3])),
+                                  fmaxf(fmaxf(xc[4], xc[5]), fmaxf(xc[6], xc[7]))),
+                            fmaxf(fmaxf(fmaxf(xc[8], xc[9]), fmaxf(xc[10], xc[11])),
+                                  fmaxf(fmaxf(xc[12], xc[13]), fmaxf(xc[14], xc[15]))));
+            float other = m;
+            swap_halves32(m, other);
+            m_blk[ct] = fmaxf(m, other) * scale_log2;
+            raise |= m_blk[ct] > m_run[ct] + kRescaleSlack;
+        }
     };
 
     // Iteration m of the main loop multiplies P(m-1) into V(m-1), turns S(m) into
@@ -295,20 +323,23 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
             // rare: raise the maximum and bring what was computed under the old
             // one (accumulators, row sum, the pending P(m-1)) to the new scale
-            const float m_new = fmaxf(m_run, m_blk);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-            l_run *= alpha;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++) acc[dt] *= alpha;
+            for (int ct = 0; ct < kColTiles; ct++) {
+                const float m_new = fmaxf(m_run[ct], m_blk[ct]);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
+                m_run[ct] = m_new;
+                l_run[ct] *= alpha;
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++)
+                for (int dt = 0; dt < 4; dt++) acc[ct][dt] *= alpha;
 #pragma unroll
-                for (int w = 0; w < 4; w++) {
-                    float lo, hi;
-                    E::unpack2(pb[ks][w], lo, hi);
-                    pb[ks][w] = E::pack2(lo * alpha, hi * alpha);
-                }
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        float lo, hi;
+                        E::unpack2(pb[ct][ks][w], lo, hi);
+                        pb[ct][ks][w] = E::pack2(lo * alpha, hi * alpha);
+                    }
+            }
         }
         // The rest of the iteration is two straight-line halves, each an MFMA
         // strand with independent vector work in its shadow:
@@ -318,12 +349,15 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         // with the masking of S(m+1), where needed, between them.  A masked score
         // is kNegBig and the maximum never drops below its start value, so masked
         // probabilities come out as exp2(-huge) = 0 without a select.
-        float s_cur[16];
-        u32x4 pb_prev[2];
-        pb_prev[0] = pb[0];
-        pb_prev[1] = pb[1];
+        float s_cur[kColTiles][16];
+        u32x4 pb_prev[kColTiles][2];
 #pragma unroll
-        for (int v = 0; v < 16; v++) s_cur[v] = x[v];
+        for (int ct = 0; ct < kColTiles; ct++) {
+            pb_prev[ct][0] = pb[ct][0];
+            pb_prev[ct][1] = pb[ct][1];
+#pragma unroll
+            for (int v = 0; v < 16; v++) s_cur[ct][v] = x[ct][v];
+        }
         // V operand: the transposing read hands each block of 16 lanes four tokens
         // of 16 consecutive dims, lane i of the block supplying the address of dims
         // 4*(i%4) .. +3 of the block's token i/4
@@ -340,29 +374,34 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
                 va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
             }
         scores();
-        {
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ct++) {
             float p[16], p_sum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[v], scale_log2, -m_run));
+                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][v], scale_log2, -m_run[ct]));
                 p_sum += p[v];
             }
-            l_run += p_sum;
+            l_run[ct] += p_sum;
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
-                pb[ks] = u32x4{E::pack2(p[8 * ks], p[8 * ks + 1]), E::pack2(p[8 * ks + 2], p[8 * ks + 3]),
-                               E::pack2(p[8 * ks + 4], p[8 * ks + 5]), E::pack2(p[8 * ks + 6], p[8 * ks + 7])};
+                pb[ct][ks] = u32x4{E::pack2(p[8 * ks], p[8 * ks + 1]), E::pack2(p[8 * ks + 2], p[8 * ks + 3]),
+                                   E::pack2(p[8 * ks + 4], p[8 * ks + 5]), E::pack2(p[8 * ks + 6], p[8 * ks + 7])};
+            // keeps P(m) in this half (it is only consumed by the next iteration)
+            asm volatile("" ::"v"(pb[ct][0]), "v"(pb[ct][1]), "v"(l_run[ct]));
         }
-        // keeps P(m) in this half (it is only consumed by the next iteration)
-        asm volatile("" ::"v"(pb[0]), "v"(pb[1]), "v"(l_run));
         if ((m + 2) * kBlock > w_mask_from) mask_scores(m + 1);   // wave-uniform
 
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) acc[dt] = E::mfma_32x32(va[dt][ks], pb_prev[ks], acc[dt]);
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ct++)
+                    acc[ct][dt] = E::mfma_32x32(va[dt][ks], pb_prev[ct][ks], acc[ct][dt]);
         block_max();
-        asm volatile("" ::"v"(m_blk));
+#pragma unroll
+        for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
     };
     for (int m = 0; m <= n_blocks; m += 4) {
         iteration(m, 0, even);
@@ -371,19 +410,21 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
         iteration(m + 3, 3, odd);
     }
 
-    float l_other = l_run;
-    swap_halves32(l_run, l_other);
-    const float l = l_run + l_other;
-    if (live) {
+#pragma unroll
+    for (int ct = 0; ct < kColTiles; ct++) {
+        float l_other = l_run[ct];
+        swap_halves32(l_run[ct], l_other);
+        const float l = l_run[ct] + l_other;
+        if (!live[ct]) continue;
         const float inv = l > 0.f ? 1.f / l : 0.f;
-        uint16_t *o = out + ((long)(q_begin + qrow) * n_qo_heads + (long)kvh * group + c_head) * kHeadDim +
+        uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
                       4 * h;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                u32x2 w = {E::pack2(acc[dt][4 * i] * inv, acc[dt][4 * i + 1] * inv),
-                           E::pack2(acc[dt][4 * i + 2] * inv, acc[dt][4 * i + 3] * inv)};
+                u32x2 w = {E::pack2(acc[ct][dt][4 * i] * inv, acc[ct][dt][4 * i + 1] * inv),
+                           E::pack2(acc[ct][dt][4 * i + 2] * inv, acc[ct][dt][4 * i + 3] * inv)};
                 *reinterpret_cast<u32x2 *>(o + dt * 32 + 8 * i) = w;
             }
     }
