@@ -191,8 +191,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
             stage_v_tile<kPageCoversTile>(lds, r, t, t_end, g, c);
             // online softmax (log2 domain)
             float m_tile = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32));
+            m_tile = quad_rows_max(m_tile);
             const float m_new = fmaxf(m_run, m_tile);
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             m_run = m_new;
@@ -229,8 +228,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
         }
 
         // ---- item epilogue
-        l_run += __shfl_xor(l_run, 16);
-        l_run += __shfl_xor(l_run, 32);
+        l_run = quad_rows_sum(l_run);
         if (c < group) {
             const int qh = kvh * group + c;
             if (item.slot < 0) {
