@@ -234,6 +234,8 @@ PREFILL_CASES = [
     ("page2", [130, 45, 7], [64, 45, 2], 2, 32, 8, 128, "bf16"),
     ("page4_group16", [200, 33], [70, 33], 4, 32, 2, 128, "f16"),
     ("long_tile", [900], [300], 16, 32, 8, 128, "bf16"),
+    ("no_kv", [0, 40], [2, 8], 16, 32, 8, 128, "bf16"),
+    ("more_queries_than_kv", [5, 33, 64], [9, 40, 64], 16, 32, 8, 128, "bf16"),
 ]
 
 
