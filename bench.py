@@ -42,6 +42,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill section")
+    ap.add_argument("--no-fragmented", action="store_true", help="skip the fragmented long-context section")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -283,6 +284,120 @@ def prefill_section(seed: int):
             "flops_per_layer": flops}
 
 
+def fragmented_section(seed: int):
+    """Baseline configuration 5 (Llama-3-70B stage, 10 layers, GQA 64q/8kv): 128 sequences with
+    lognormal context lengths on a pool fragmented by evictions (40 % of the pages freed and
+    handed out again, lowest id first); 25 % of the sequences are swapped out and back in
+    (per-request offload / reload of scattered pages), then decode steps run."""
+    import numpy as np
+    import torch
+
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.kvcache.manager import KVCacheManager
+    from deserve_amd.kvcache.paged.chunk_pool import CpuChunkPool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.kvcache.virtual import VirtualPagedKVCache, VirtualPagePool
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.paged_ops import append_paged_kv_cache
+    from deserve_amd.synthetic import config5_context_lengths, fill_normal
+    from deserve_amd.task import SamplingParams, TaskData
+
+    dev = torch.device("cuda")
+    L, P, Hq, Hkv, D, B, steps = 10, 16, 64, 8, 128, 128, 6
+    rng = np.random.default_rng(seed + 50)
+    ctx_lens = config5_context_lengths(seed + 3)
+    need = int((-(-(ctx_lens + steps + 8) // P)).sum())
+    pool = VirtualPagePool(L, int(need / 0.4 * 1.05) + 128, 0, P, dev, torch.bfloat16)
+    fill_normal(pool.pages, seed + 51)
+    rows = PageTableAllocator(B + 40, 32768 + 64, P, dev)
+    filler = pool.alloc(pool.num_avails)
+    pool.free(torch.from_numpy(rng.permutation(filler.numpy())[: int(0.4 * len(filler))].copy()))
+    made = {}
+    for b in rng.permutation(B):                        # out-of-order arrival into the holes
+        c = VirtualPagedKVCache.empty(rows, pool)
+        c.extend(int(ctx_lens[b]))
+        made[int(b)] = c
+    tasks = [TaskData(f"f{b}", int(ctx_lens[b]), 1, 1, int(ctx_lens[b]), SamplingParams()) for b in range(B)]
+    caches = [made[b] for b in range(B)]
+    mgr = KVCacheManager(pool, CpuChunkPool(L, 15, P, torch.bfloat16), rows)
+    swapped = sorted(rng.choice(B, size=B // 4, replace=False).tolist())
+    page_bytes = 2 * P * Hkv * D * 2
+    swap_bytes = sum(caches[b].page_table.occupied for b in swapped) * L * page_bytes
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        mgr.synchronize()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    handles = []
+    t_out = timed(lambda: handles.extend(mgr.copy_gpu_to_cpu(caches[b], tasks[b].task_id) for b in swapped))
+    for b in swapped:
+        caches[b].free()
+    back = []
+    t_in = timed(lambda: back.extend(mgr.copy_cpu_to_gpu(h, tasks[b].task_id) for h, b in zip(handles, swapped)))
+    for h in handles:
+        h.free()
+    for b, c in zip(swapped, back):
+        caches[b] = c
+
+    gen = torch.Generator(device="cuda").manual_seed(seed + 52)
+    mk = lambda h: torch.randn((L, B, h, D), generator=gen, device=dev).to(torch.bfloat16)
+    q, k, v = mk(Hq), mk(Hkv), mk(Hkv)
+    w, _ = get_wrappers(dev)
+    ev, attn_bytes = [], 0
+
+    def decode_step(record: bool):
+        nonlocal attn_bytes
+        c = FlashDecodeCtx.init_paged_decode_ctx(tasks, caches, w)
+        w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
+                        last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
+                        head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
+                        last_page_len_host=c.host["kv_last_page_lens"])
+        for layer in range(L):
+            pages = pool.get_layered_pages(layer)
+            append_paged_kv_cache(k[layer], v[layer], c.indptr, pages, c.kv_page_indices,
+                                  c.kv_page_indptr, c.kv_last_page_lens)
+            if record and layer % 2 == 0:
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                out = w.forward(q[layer], pages, phases=1)
+                e.record()
+                w.forward(q[layer], pages, phases=2, out=out)
+                ev.append((s, e))
+            else:
+                w.forward(q[layer], pages)
+        w.end_forward()
+        if record:
+            kv_lens = np.array([t.start_pos + 1 for t in tasks], dtype=np.int64)
+            attn_bytes = attention_bytes_per_layer(kv_lens, int(c.host["kv_page_indptr"][-1]), B, Hq, D, 2,
+                                                   2 * Hkv * D * 2)
+        for t in tasks:
+            t.step()
+
+    for _ in range(2):
+        decode_step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps - 2):
+        decode_step(True)
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) / (steps - 2) * 1e3
+    us = sorted(s.elapsed_time(e) for s, e in ev)
+    attn_us = us[len(us) // 2] * 1e3
+    return {"workload": "BASELINE.json configs[4]: 10 layers, bf16, GQA 64q/8kv, page 16, 128 sequences, "
+                        "lognormal ctx (median 2048, [64,32768]), 40 % of the pool freed and reallocated out "
+                        "of order; 32 sequences swapped out and back in before the decode steps",
+            "kv_tokens": int(sum(t.start_pos for t in tasks)),
+            "swap_out_GBps": round(swap_bytes / t_out / 1e9, 2), "swap_in_GBps": round(swap_bytes / t_in / 1e9, 2),
+            "swapped_bytes": swap_bytes, "decode_ms_per_step": round(ms_step, 3),
+            "attention_us_per_layer": round(attn_us, 1),
+            "attention_GBps": round(attn_bytes / attn_us / 1e3, 1),
+            "attention_frac_of_hbm_peak": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+
 def main() -> int:
     a = parse_args()
     if a.gpus != 1:
@@ -417,6 +532,9 @@ def main() -> int:
         torch.cuda.empty_cache()
     if not a.no_prefill:
         out["prefill"] = prefill_section(a.seed)
+        torch.cuda.empty_cache()
+    if not a.no_fragmented:
+        out["fragmented"] = fragmented_section(a.seed)
     print(json.dumps(out))
     return 0
 
