@@ -260,6 +260,64 @@ def test_prefill_attention_matches_oracle(case):
     w.end_forward()
 
 
+def test_prefill_attention_random_shapes():
+    """Seeded sweep over page sizes, GQA groups, dtypes and ragged (kv, chunk) lengths,
+    including requests with fewer kv tokens than queries."""
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+
+    rng = np.random.default_rng(77)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    done = 0
+    while done < 40:
+        P = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        Hq = Hkv * int(rng.choice([1, 2, 4, 8, 16, 32]))
+        if Hq > 64:
+            continue
+        dtype = str(rng.choice(["bf16", "f16"]))
+        qo = [int(rng.integers(0, 140)) for _ in range(int(rng.integers(1, 5)))]
+        kv = [int(n + rng.integers(0, 300)) if rng.random() < 0.85 else int(rng.integers(0, n + 1)) for n in qo]
+        if sum(qo) == 0:
+            continue
+        causal = bool(rng.integers(0, 2))
+        _announce("prefill random", P, Hq, Hkv, dtype, kv, qo, causal)
+        sc = make_scenario(2000 + done, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
+        w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                        _dev_i32(sc.kv_last_page_lens), Hq, Hkv, 128, P)
+        out = w.forward(to_torch(sc.q, dtype), to_torch(sc.pages, dtype), causal=causal)
+        w.end_forward()
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
+                                     sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
+        assert np.isfinite(got).all()
+        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, qo, causal)
+        done += 1
+
+
+def test_decode_attention_random_shapes():
+    """Seeded sweep over page sizes, GQA groups, dtypes, batch and workgroup counts."""
+    rng = np.random.default_rng(78)
+    done = 0
+    while done < 40:
+        P = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        Hkv = int(rng.choice([1, 2, 4, 8]))
+        Hq = Hkv * int(rng.choice([1, 2, 4, 8, 16]))
+        if Hq > 64:
+            continue
+        dtype = str(rng.choice(["bf16", "f16"]))
+        kv = [int(rng.integers(1, 1200)) for _ in range(int(rng.integers(1, 9)))]
+        target = int(rng.choice([0, 1, 3, 16, 100]))
+        _announce("decode random", P, Hq, Hkv, dtype, kv, target)
+        sc = make_scenario(3000 + done, kv_lens=kv, qo_lens=[1] * len(kv), P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
+        got, _ = _run_decode(sc, target)
+        want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                    sc.kv_last_page_lens, dtype)
+        assert np.isfinite(got).all()
+        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, target)
+        done += 1
+
+
 def test_prefill_with_one_query_equals_decode():
     from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
 
