@@ -2,13 +2,15 @@
 // query i of the n_b new tokens of request b sees kv positions j <= kv_len_b - n_b + i.
 //
 // Bound: MFMA for long chunks.  Work decomposition: one workgroup = one kv head x
-// one tile of query rows; each of its waves owns 32 columns, a column being a
-// (query position, q head of the GQA group) pair, so the MFMA N dimension is
-// dense.  The workgroup walks the request's K/V in blocks of 32 tokens that its
-// waves load together (each a few rows) into a double-buffered LDS stage, so a
+// one tile of query rows; each of its waves owns 32 columns (kColTiles tiles of
+// 32), a column being a (query position, q head of the GQA group) pair, so the
+// MFMA N dimension is dense.  The workgroup walks the request's K/V in blocks of
+// 32 tokens that its waves load together (each a few rows) into LDS stages, so a
 // K/V byte crosses the vector memory path once per workgroup instead of once per
 // wave: with every wave streaming K/V on its own the kernel was bound by that
-// path at a sixth of the MFMA rate.
+// path at a sixth of the MFMA rate.  Row pitches of 272 (K) and 320 (V) bytes keep
+// the operand reads free of LDS bank conflicts (SQ_LDS_BANK_CONFLICT = 0; 288 for
+// either costs 4 %).
 //
 // All products use the 32x32x16 MFMA (measured on MI355X at 2.2 PFLOP/s bf16,
 // against 1.3 PFLOP/s for 16x16x32).  Per block a wave computes S^T = K.Q^T
@@ -33,10 +35,10 @@ namespace dskv {
 #ifndef DSKV_PREFILL_VPITCH
 #define DSKV_PREFILL_VPITCH 320
 #endif
-constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
 #ifndef DSKV_PREFILL_COLTILES
 #define DSKV_PREFILL_COLTILES 1
 #endif
+constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
 constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
 constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
 constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
