@@ -526,10 +526,13 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
     *p++ = (int32_t)wgs;
     *p++ = n_slots;
     *p++ = batch;
-    p = std::copy(reinterpret_cast<const int32_t *>(items.data()),
-                  reinterpret_cast<const int32_t *>(items.data()) + items.size() * kItemWords, p);
+    // the variable-length part (the items) goes last, so that where everything lies
+    // depends only on the batch and the number of workgroups: a captured launch
+    // stays valid from step to step
     p = std::copy(wg_ptr.begin(), wg_ptr.end(), p);
-    std::copy(req.begin(), req.end(), p);
+    p = std::copy(req.begin(), req.end(), p);
+    std::copy(reinterpret_cast<const int32_t *>(items.data()),
+              reinterpret_cast<const int32_t *>(items.data()) + items.size() * kItemWords, p);
     *n_items_out = (int32_t)items.size();
     *n_workgroups_out = (int32_t)wgs;
     *plan_words_out = words;
@@ -574,9 +577,9 @@ extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pag
                  "decode_attn: workspace (%lld bytes) too small for %d items of %d requests",
                  (long long)workspace_bytes, n_items, batch);
 
-    const Item *items = reinterpret_cast<const Item *>(plan_dev + kPlanHeaderWords);
-    const int32_t *wg_ptr = plan_dev + kPlanHeaderWords + (int64_t)n_items * kItemWords;
+    const int32_t *wg_ptr = plan_dev + kPlanHeaderWords;
     const int32_t *req_parts = wg_ptr + n_workgroups + 1;
+    const Item *items = reinterpret_cast<const Item *>(req_parts + 2 * (int64_t)batch);
     // slots are numbered densely from 0, so part_ml can sit after max_slots O blocks
     float *part_o = reinterpret_cast<float *>(workspace);
     float *part_ml = part_o ? part_o + max_slots * n_qo_heads * (int64_t)head_dim : nullptr;

@@ -1,0 +1,77 @@
+"""A decode step of a stage as a replayed HIP graph.
+
+The reference launches every kernel of every layer from Python each step; at
+decode sizes the step is a few dozen short launches.  ``GraphedDecodeStep``
+captures what ``layer_storage.forward(xs, ctx)`` launches for one batch shape
+into a graph and replays it: per step the host only rebuilds the CSR metadata
+and the split-KV work list in pinned buffers that never move, copies both to
+device buffers that never move, and replays.  A new batch size (or workgroup
+count) triggers a new capture.
+
+Nothing that is captured clears memory with a memset node, and the library
+calls allocate nothing; the outputs of the captured forward live in the graph's
+own memory pool and are overwritten by every replay.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from deserve_amd import _lib
+from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+from deserve_amd.model.context.flash import FlashDecodeCtx, MetadataBuffers
+from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+from deserve_amd.task import TaskData
+
+
+class GraphedDecodeStep:
+    def __init__(self, layer_storage, wrapper: BatchDecodeWithPagedKVCacheWrapper, max_batch: int,
+                 max_pages: int, device: torch.device, num_qo_heads: int, num_kv_heads: int,
+                 head_dim: int, page_size: int, target_workgroups: int = 0) -> None:
+        self.layer_storage, self.wrapper = layer_storage, wrapper
+        self.shape = dict(num_qo_heads=num_qo_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
+                          page_size=page_size)
+        self.target_workgroups = target_workgroups
+        self.meta = MetadataBuffers(max_batch, max_pages, device)
+        words = int(_lib.lib().dskv_decode_plan_bound(max_batch, max_pages * page_size))
+        self.plan = (torch.empty((words,), dtype=torch.int32, pin_memory=True),
+                     torch.empty((words,), dtype=torch.int32, device=device))
+        self._key = None
+        self._graph = None
+        self._inputs: List[torch.Tensor] = []
+        self._output = None
+        self.captures = 0
+
+    def _prepare(self, task_datas: Sequence[TaskData], kvcaches: Sequence[PagedKVCache]) -> FlashDecodeCtx:
+        ctx = FlashDecodeCtx.init_paged_decode_ctx(list(task_datas), list(kvcaches), self.wrapper, self.meta)
+        self.wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ctx.kv_page_indices,
+                                   last_page_len=ctx.kv_last_page_lens,
+                                   indptr_host=ctx.host["kv_page_indptr"],
+                                   last_page_len_host=ctx.host["kv_last_page_lens"],
+                                   target_workgroups=self.target_workgroups, plan_buffers=self.plan,
+                                   **self.shape)
+        return ctx
+
+    def run(self, xs, task_datas: Sequence[TaskData], kvcaches: Sequence[PagedKVCache]) -> torch.Tensor:
+        """xs: a tensor or a tuple of tensors, as the stage's forward takes them.  Returns the
+        stage's output (valid until the next run)."""
+        tensors = list(xs) if isinstance(xs, (tuple, list)) else [xs]
+        ctx = self._prepare(task_datas, kvcaches)
+        w = self.wrapper
+        key = (len(task_datas), w._n_workgroups, w._n_items > len(task_datas),
+               tuple((tuple(t.shape), t.dtype) for t in tensors))
+        if key != self._key:
+            self._inputs = [t.clone() for t in tensors]
+            static = tuple(self._inputs) if isinstance(xs, (tuple, list)) else self._inputs[0]
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self._output = self.layer_storage.forward(static, ctx)
+            self._graph, self._key = graph, key
+            self.captures += 1
+        else:
+            for dst, src in zip(self._inputs, tensors):
+                dst.copy_(src, non_blocking=True)
+        self._graph.replay()
+        w.end_forward()
+        return self._output

@@ -57,7 +57,20 @@ def build_host_metadata(task_datas: Sequence[TaskData],
                 seqlens=seqlens, kv_page_indices=indices)
 
 
-def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device):
+class MetadataBuffers:
+    """A pinned and a device int32 buffer that stay where they are from step to step, for
+    callers that replay captured launches (the kernels then find the metadata at the same
+    addresses every step).  The batch-sized arrays come first, the block-table entries last,
+    so only the batch decides where an array starts."""
+
+    def __init__(self, max_batch: int, max_pages: int, device: torch.device) -> None:
+        words = 5 * ((max_batch + 1 + 3) // 4 * 4) + (max_pages + 3) // 4 * 4
+        self.host = torch.empty((words,), dtype=torch.int32, pin_memory=True)
+        self.dev = torch.empty((words,), dtype=torch.int32, device=device)
+
+
+def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
+                    buffers: "MetadataBuffers | None" = None):
     """One pinned staging buffer, one async copy; returns (device views, host views)."""
     sizes = [meta[f].shape[0] for f in _FIELDS]
     # each array starts on a 16-byte boundary
@@ -66,11 +79,20 @@ def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device):
         starts.append(total)
         total += (n + 3) // 4 * 4
     use_gpu = torch.device(device).type == "cuda"
-    staging = torch.empty((max(total, 4),), dtype=torch.int32, pin_memory=use_gpu)
+    if buffers is not None:
+        if total > buffers.host.numel():
+            raise ValueError(f"step metadata needs {total} words, the buffers hold {buffers.host.numel()}")
+        staging = buffers.host
+    else:
+        staging = torch.empty((max(total, 4),), dtype=torch.int32, pin_memory=use_gpu)
     host_np = staging.numpy()
     for f, s, n in zip(_FIELDS, starts, sizes):
         host_np[s: s + n] = meta[f]
-    dev = staging.to(device, non_blocking=True) if use_gpu else staging
+    if buffers is not None:
+        dev = buffers.dev
+        dev[:total].copy_(staging[:total], non_blocking=True)
+    else:
+        dev = staging.to(device, non_blocking=True) if use_gpu else staging
     dev_views = {f: dev[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
     host_views = {f: staging[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
     return dev_views, host_views
@@ -86,9 +108,10 @@ class FlashForwardCtx(PagedForwardCtx):
 
     @classmethod
     def init_paged_forward_ctx(cls, task_datas: List[TaskData],
-                               kvcaches: List[PagedKVCache[GpuPagePool]], **extra):
+                               kvcaches: List[PagedKVCache[GpuPagePool]],
+                               buffers: "MetadataBuffers | None" = None, **extra):
         pool = kvcaches[0].pool
-        dev, host = upload_metadata(build_host_metadata(task_datas, kvcaches), pool.main_device)
+        dev, host = upload_metadata(build_host_metadata(task_datas, kvcaches), pool.main_device, buffers)
         return cls(bsz=len(task_datas), seqlens=dev["seqlens"], layer_id=0, page_pool=pool,
                    offsets=dev["offsets"], indptr=dev["indptr"],
                    kv_page_indices=dev["kv_page_indices"], kv_page_indptr=dev["kv_page_indptr"],
@@ -102,8 +125,9 @@ class FlashDecodeCtx(FlashForwardCtx):
     @classmethod
     def init_paged_decode_ctx(cls, task_datas: List[TaskData],
                               kvcaches: List[PagedKVCache[GpuPagePool]],
-                              wrapper: BatchDecodeWithPagedKVCacheWrapper) -> "FlashDecodeCtx":
-        return cls.init_paged_forward_ctx(task_datas, kvcaches, decode_wrapper=wrapper)
+                              wrapper: BatchDecodeWithPagedKVCacheWrapper,
+                              buffers: "MetadataBuffers | None" = None) -> "FlashDecodeCtx":
+        return cls.init_paged_forward_ctx(task_datas, kvcaches, buffers, decode_wrapper=wrapper)
 
 
 @dataclass

@@ -116,7 +116,9 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
                       last_page_len: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, *, indptr_host: Optional[torch.Tensor] = None,
                       last_page_len_host: Optional[torch.Tensor] = None,
-                      target_workgroups: int = 0, **_ignored) -> None:
+                      target_workgroups: int = 0, plan_buffers=None, **_ignored) -> None:
+        """plan_buffers: optional (pinned int32, device int32) pair that receives the work
+        list instead of fresh tensors, for callers that replay captured launches."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._indptr, self._indices = _i32(indptr), _i32(indices)
         h_indptr = self._host(indptr, indptr_host)
@@ -125,7 +127,12 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         L = _lib.lib()
         total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
         cap = L.dskv_decode_plan_bound(batch, total_tokens)
-        plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
+        if plan_buffers is not None:
+            plan = plan_buffers[0]
+            if plan.numel() < cap:
+                raise ValueError(f"plan buffer holds {plan.numel()} words, {cap} may be needed")
+        else:
+            plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
         n_items, n_wgs = ctypes.c_int32(), ctypes.c_int32()
         words, ws = ctypes.c_int64(), ctypes.c_int64()
         rc = L.dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, page_size,
@@ -137,7 +144,11 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
         self._plan_host = plan                       # keep alive until the upload has run
-        self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
+        if plan_buffers is not None:
+            self._plan = plan_buffers[1]
+            self._plan[: max(words.value, 1)].copy_(plan[: max(words.value, 1)], non_blocking=True)
+        else:
+            self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
         self._planned = True
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,

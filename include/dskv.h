@@ -71,9 +71,10 @@ int dskv_scatter_pages(void *pool, const void *chunk, const int32_t *page_ids, i
  * dskv_decode_plan runs on the host from host copies of the CSR metadata.  It
  * lays all requests' 16-token tiles end to end, cuts the sequence into one equal
  * share per workgroup and writes the resulting work list to plan_host (int32
- * words: 4 header words, 8 per item, n_workgroups + 1 share offsets, 2 per
- * request); the caller copies it to the device once per step and reuses it for
- * every layer.
+ * words: 4 header words, n_workgroups + 1 share offsets, 2 per request, then 8
+ * per item - the variable-length part last, so that the layout depends only on
+ * the batch and the number of workgroups); the caller copies it to the device
+ * once per step and reuses it for every layer.
  *   target_workgroups:   <= 0 = one per compute unit of the current device.
  *   plan_capacity_words: size of plan_host; dskv_decode_plan_bound(batch,
  *                        total_tokens) words always suffice.

@@ -71,9 +71,10 @@ def _plan(lens, P=16, Hq=32, Hkv=8, D=128, target=0):
                               ctypes.byref(words), ctypes.byref(ws))
     assert rc == 0, _lib.last_error()
     assert plan[:4].tolist()[:2] == [n.value, wgs.value] and plan[3] == len(lens)
-    items = plan[4: 4 + n.value * 8].reshape(-1, 8)
-    wg_ptr = plan[4 + n.value * 8: 4 + n.value * 8 + wgs.value + 1]
-    req = plan[4 + n.value * 8 + wgs.value + 1: words.value].reshape(-1, 2)
+    wg_ptr = plan[4: 4 + wgs.value + 1]
+    req = plan[4 + wgs.value + 1: 4 + wgs.value + 1 + 2 * len(lens)].reshape(-1, 2)
+    items = plan[4 + wgs.value + 1 + 2 * len(lens): words.value].reshape(-1, 8)
+    assert items.shape[0] == n.value
     assert np.array_equal(items[:, 4], indptr[items[:, 0]])          # page_begin = kv_page_indptr[b]
     return items[:, :4], wg_ptr, req, ws.value, int(plan[2])
 

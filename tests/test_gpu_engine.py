@@ -227,3 +227,61 @@ def test_scheduler_policies_under_page_pressure(policy):
     sched.synchronize()
     assert finished == set(prompt_len), (finished, decoded)
     assert offloads > 0 and reloads > 0, (offloads, reloads)
+
+
+def test_graphed_decode_step_matches_eager_steps():
+    """The decode step replayed as a HIP graph gives, step after step, the bits of the eager
+    step: contexts grow across page boundaries between replays (new block-table entries, a
+    new work list), eager launches run between replays, and a different batch re-captures."""
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.execution.graph import GraphedDecodeStep
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.stage import KVStage, StageArgs
+    from deserve_amd.synthetic import make_decode_workload
+
+    print("[case] graphed decode step", flush=True)
+    Lg, B = 3, 6
+    lens = np.array([13, 16, 300, 47, 1000, 31])
+    args = dict(n_heads=HQ, n_kv_heads=HKV, dim=HQ * D, page_size=P, n_layers=Lg)
+
+    def fresh(batch_lens, seed):
+        return make_decode_workload("g", batch_lens, Lg, HQ, HKV, D, P, torch.bfloat16,
+                                    headroom_tokens=64, seed=seed, fill=True)
+
+    wl_e, wl_g = fresh(lens, 11), fresh(lens, 11)          # identical twins: eager and graphed
+    assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16))
+    stage = KVStage(StageArgs(**args), use_rope=True)
+    wrapper, _ = get_wrappers(DEV)
+    gwrapper = type(wrapper)(torch.empty(32 << 20, dtype=torch.uint8, device=DEV))
+    step = GraphedDecodeStep(stage, gwrapper, max_batch=8, max_pages=4096, device=DEV,
+                             num_qo_heads=HQ, num_kv_heads=HKV, head_dim=D, page_size=P,
+                             target_workgroups=16)     # fixed: with fewer tiles than CUs the count would follow the tiles
+
+    def eager(wl, xs):
+        ctx = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, wrapper)
+        wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ctx.kv_page_indices,
+                              last_page_len=ctx.kv_last_page_lens, num_qo_heads=HQ, num_kv_heads=HKV,
+                              head_dim=D, page_size=P, indptr_host=ctx.host["kv_page_indptr"],
+                              last_page_len_host=ctx.host["kv_last_page_lens"], target_workgroups=16)
+        out = stage.forward(xs, ctx)
+        wrapper.end_forward()
+        return out
+
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    for it in range(8):                                    # 8 tokens: requests 1, 3 and 5 open new pages
+        n = len(wl_e.tasks)
+        xs = tuple(torch.randn((Lg, n, h, D), device=DEV, generator=gen).to(torch.bfloat16)
+                   for h in (HQ, HKV, HKV))
+        want = eager(wl_e, xs).clone()
+        got = step.run(xs, wl_g.tasks, wl_g.caches).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), it
+        assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16)), it
+        for wl in (wl_e, wl_g):
+            for t in wl.tasks:
+                t.step()
+        if it == 4:                                        # a request leaves: smaller batch, new capture
+            for wl in (wl_e, wl_g):
+                wl.caches.pop(2).free()
+                wl.tasks.pop(2)
+    assert step.captures == 2
