@@ -43,6 +43,7 @@ def parse_args():
     ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill section")
     ap.add_argument("--no-fragmented", action="store_true", help="skip the fragmented long-context section")
+    ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--section", choices=["swap", "fragmented"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -443,7 +444,8 @@ def main() -> int:
         _lib.build()
     torch.cuda.set_device(0)
     L, Hq, Hkv, D, P = 16, 32, 8, 128, 16
-    total_steps = a.steps + a.warmup
+    graph_steps = 0 if a.no_graph else 24
+    total_steps = a.steps + a.warmup + graph_steps
     ctx = config2_context_lengths(a.seed)
     wl = make_decode_workload("cfg2", ctx, L, Hq, Hkv, D, P, torch.bfloat16,
                               headroom_tokens=total_steps + 8, seed=a.seed, use_rope=a.rope)
@@ -551,6 +553,34 @@ def main() -> int:
                            "avg_launch_us": round(avg_ms * 1e3, 2), "launches": len(times_ms),
                            "intervals_left_out": len(all_ms) - len(times_ms),
                            "algorithmic_bytes_per_launch": int(sum(attn_bytes_layer) / len(attn_bytes_layer))}
+    if graph_steps:
+        # the same step (rope off: append + attention per layer through the stage) captured
+        # once into a HIP graph and replayed; per step the host rebuilds metadata and plan only
+        from deserve_amd.execution.graph import GraphedDecodeStep
+        gstep = GraphedDecodeStep(wl.stage, decode_wrapper, max_batch=wl.batch,
+                                  max_pages=int(last_ctx.host["kv_page_indptr"][-1]) + 4 * wl.batch,
+                                  device=wl.pool.main_device, num_qo_heads=Hq, num_kv_heads=Hkv,
+                                  head_dim=D, page_size=P, target_workgroups=a.workgroups)
+        xs = (wl.q, wl.k, wl.v)
+
+        def graphed():
+            gstep.run(xs, wl.tasks, wl.caches)
+            for t in wl.tasks:
+                t.step()
+
+        for _ in range(4):
+            graphed()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(graph_steps - 4):
+            graphed()
+        torch.cuda.synchronize()
+        g_ms = (time.perf_counter() - t0) / (graph_steps - 4) * 1e3
+        out["graph"] = {"ms_per_step": round(g_ms, 4),
+                        "value_GBps": round(step_bytes[-1] / g_ms / 1e6, 1),
+                        "pct_of_hbm_peak": round(100.0 * step_bytes[-1] / g_ms / 1e6 / HBM_PEAK_GBPS, 2),
+                        "captures": gstep.captures,
+                        "note": "same step replayed as one HIP graph (host: metadata + plan only)"}
     if not a.no_cpu_baseline:
         meta = {n: last_ctx.host[n].numpy() for n in ("kv_page_indices", "kv_page_indptr", "kv_last_page_lens")}
         out["cpu_baseline"] = cpu_baseline(wl, meta, sample_requests=16)

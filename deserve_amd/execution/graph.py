@@ -20,7 +20,7 @@ import torch
 
 from deserve_amd import _lib
 from deserve_amd.kvcache.paged.kvcache import PagedKVCache
-from deserve_amd.model.context.flash import FlashDecodeCtx, MetadataBuffers
+from deserve_amd.model.context.flash import FlashDecodeCtx, MetadataBuffers, StagedUpload
 from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
 from deserve_amd.task import TaskData
 
@@ -35,8 +35,7 @@ class GraphedDecodeStep:
         self.target_workgroups = target_workgroups
         self.meta = MetadataBuffers(max_batch, max_pages, device)
         words = int(_lib.lib().dskv_decode_plan_bound(max_batch, max_pages * page_size))
-        self.plan = (torch.empty((words,), dtype=torch.int32, pin_memory=True),
-                     torch.empty((words,), dtype=torch.int32, device=device))
+        self.plan = StagedUpload(words, device)
         self._key = None
         self._graph = None
         self._inputs: List[torch.Tensor] = []

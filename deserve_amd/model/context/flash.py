@@ -57,16 +57,43 @@ def build_host_metadata(task_datas: Sequence[TaskData],
                 seqlens=seqlens, kv_page_indices=indices)
 
 
-class MetadataBuffers:
-    """A pinned and a device int32 buffer that stay where they are from step to step, for
-    callers that replay captured launches (the kernels then find the metadata at the same
-    addresses every step).  The batch-sized arrays come first, the block-table entries last,
-    so only the batch decides where an array starts."""
+class StagedUpload:
+    """An int32 device buffer that stays where it is from step to step, fed through pinned
+    staging: for callers that replay captured launches (the kernels then find their inputs
+    at the same addresses every step).  The copy to the device is asynchronous, so the
+    staging a step fills must not be the one an earlier, still pending copy reads from:
+    there are two, used in turn, and a staging buffer is handed out again only after the
+    copy that last read it has run."""
+
+    def __init__(self, words: int, device: torch.device) -> None:
+        self.dev = torch.empty((words,), dtype=torch.int32, device=device)
+        self._host = [torch.empty((words,), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._copied = [torch.cuda.Event(), torch.cuda.Event()]
+        self._pending = [False, False]
+        self._turn = 0
+
+    def staging(self) -> torch.Tensor:
+        """The pinned buffer to fill for the next upload (waits for its previous copy)."""
+        self._turn ^= 1
+        if self._pending[self._turn]:
+            self._copied[self._turn].synchronize()
+            self._pending[self._turn] = False
+        return self._host[self._turn]
+
+    def upload(self, words: int) -> None:
+        """Enqueues the copy of the first `words` words of the current staging buffer."""
+        t = self._turn
+        self.dev[:words].copy_(self._host[t][:words], non_blocking=True)
+        self._copied[t].record()
+        self._pending[t] = True
+
+
+class MetadataBuffers(StagedUpload):
+    """StagedUpload sized for the six CSR arrays of a step.  The batch-sized arrays come
+    first, the block-table entries last, so only the batch decides where an array starts."""
 
     def __init__(self, max_batch: int, max_pages: int, device: torch.device) -> None:
-        words = 5 * ((max_batch + 1 + 3) // 4 * 4) + (max_pages + 3) // 4 * 4
-        self.host = torch.empty((words,), dtype=torch.int32, pin_memory=True)
-        self.dev = torch.empty((words,), dtype=torch.int32, device=device)
+        super().__init__(5 * ((max_batch + 1 + 3) // 4 * 4) + (max_pages + 3) // 4 * 4, device)
 
 
 def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
@@ -80,9 +107,9 @@ def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
         total += (n + 3) // 4 * 4
     use_gpu = torch.device(device).type == "cuda"
     if buffers is not None:
-        if total > buffers.host.numel():
-            raise ValueError(f"step metadata needs {total} words, the buffers hold {buffers.host.numel()}")
-        staging = buffers.host
+        if total > buffers.dev.numel():
+            raise ValueError(f"step metadata needs {total} words, the buffers hold {buffers.dev.numel()}")
+        staging = buffers.staging()
     else:
         staging = torch.empty((max(total, 4),), dtype=torch.int32, pin_memory=use_gpu)
     host_np = staging.numpy()
@@ -90,7 +117,7 @@ def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
         host_np[s: s + n] = meta[f]
     if buffers is not None:
         dev = buffers.dev
-        dev[:total].copy_(staging[:total], non_blocking=True)
+        buffers.upload(total)
     else:
         dev = staging.to(device, non_blocking=True) if use_gpu else staging
     dev_views = {f: dev[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}

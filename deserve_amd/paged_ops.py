@@ -117,8 +117,9 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
                       head_dim: int, page_size: int, *, indptr_host: Optional[torch.Tensor] = None,
                       last_page_len_host: Optional[torch.Tensor] = None,
                       target_workgroups: int = 0, plan_buffers=None, **_ignored) -> None:
-        """plan_buffers: optional (pinned int32, device int32) pair that receives the work
-        list instead of fresh tensors, for callers that replay captured launches."""
+        """plan_buffers: optional staged upload (an object with staging() / upload(words) /
+        dev, see model.context.flash.StagedUpload) that receives the work list instead of
+        fresh tensors, for callers that replay captured launches."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._indptr, self._indices = _i32(indptr), _i32(indices)
         h_indptr = self._host(indptr, indptr_host)
@@ -128,9 +129,9 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
         cap = L.dskv_decode_plan_bound(batch, total_tokens)
         if plan_buffers is not None:
-            plan = plan_buffers[0]
-            if plan.numel() < cap:
-                raise ValueError(f"plan buffer holds {plan.numel()} words, {cap} may be needed")
+            if plan_buffers.dev.numel() < cap:
+                raise ValueError(f"plan buffer holds {plan_buffers.dev.numel()} words, {cap} may be needed")
+            plan = plan_buffers.staging()
         else:
             plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
         n_items, n_wgs = ctypes.c_int32(), ctypes.c_int32()
@@ -145,8 +146,8 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
         self._plan_host = plan                       # keep alive until the upload has run
         if plan_buffers is not None:
-            self._plan = plan_buffers[1]
-            self._plan[: max(words.value, 1)].copy_(plan[: max(words.value, 1)], non_blocking=True)
+            self._plan = plan_buffers.dev
+            plan_buffers.upload(max(words.value, 1))
         else:
             self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
         self._planned = True

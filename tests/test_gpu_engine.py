@@ -246,7 +246,7 @@ def test_graphed_decode_step_matches_eager_steps():
 
     def fresh(batch_lens, seed):
         return make_decode_workload("g", batch_lens, Lg, HQ, HKV, D, P, torch.bfloat16,
-                                    headroom_tokens=64, seed=seed, fill=True)
+                                    headroom_tokens=96, seed=seed, fill=True)
 
     wl_e, wl_g = fresh(lens, 11), fresh(lens, 11)          # identical twins: eager and graphed
     assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16))
@@ -284,4 +284,19 @@ def test_graphed_decode_step_matches_eager_steps():
             for wl in (wl_e, wl_g):
                 wl.caches.pop(2).free()
                 wl.tasks.pop(2)
+    assert step.captures == 2
+    # the host running ahead of the GPU: steps enqueued back to back, no synchronisation
+    # between them (the staging of a step must not be refilled under a pending copy)
+    for it in range(20):
+        n = len(wl_e.tasks)
+        xs = tuple(torch.randn((Lg, n, h, D), device=DEV, generator=gen).to(torch.bfloat16)
+                   for h in (HQ, HKV, HKV))
+        want = eager(wl_e, xs)
+        got = step.run(xs, wl_g.tasks, wl_g.caches)
+        for wl in (wl_e, wl_g):
+            for t in wl.tasks:
+                t.step()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16))
     assert step.captures == 2
