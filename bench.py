@@ -196,9 +196,15 @@ def swap_section(seed: int):
     with torch.cuda.stream(side):
         eng.fence()                 # the side stream (not the compute stream) waits for the swap
         done.record()
+    # a stage hands every step's output on before it starts the next but one: at most two
+    # steps are queued on the GPU at any time
     steps = 0
+    in_flight = [torch.cuda.Event(), torch.cuda.Event()]
     while not done.query():
+        if steps >= 2:
+            in_flight[steps % 2].synchronize()
         decode_step()
+        in_flight[steps % 2].record()
         steps += 1
     done.synchronize()
     t_swap = time.perf_counter() - t0

@@ -52,6 +52,7 @@ _SIGNATURES = {
                                   c_void_p]),
     "dskv_rope_append_paged_kv": (c_int32, [c_void_p] * 10 + [c_int32] * 6 + [c_float, c_int32,
                                                                         c_void_p]),
+    "dskv_upload_words": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "dskv_swap_slice": (c_int32, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
     "dskv_swap_create": (c_int32, [POINTER(c_void_p), c_int64]),

@@ -68,7 +68,42 @@ static int move_pages(bool gather, void *pool, void *chunk, const int32_t *page_
     return 0;
 }
 
+// Small host-to-device upload done by a kernel: every lane reads 16 bytes of
+// pinned host memory over the link and stores them to HBM.  For the few tens
+// of KiB of per-step metadata this takes microseconds, and unlike an async
+// memcpy it stays on the compute queue of the caller's stream: a copy engine
+// between two kernels of a stream costs a hand-over to the engine and one
+// back, and with a host that runs several steps ahead those hand-overs have
+// been measured to stall whole steps.
+__global__ __launch_bounds__(256) void upload_words_kernel(uint32_t *__restrict__ dst,
+                                                           const uint32_t *__restrict__ src,
+                                                           long n_words)
+{
+    const long quads = n_words / 4;
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < quads)
+        reinterpret_cast<u32x4 *>(dst)[i] = reinterpret_cast<const u32x4 *>(src)[i];
+    else if (i == quads)
+        for (long w = quads * 4; w < n_words; w++) dst[w] = src[w];
+}
+
 }  // namespace dskv
+
+extern "C" int dskv_upload_words(void *dst, const void *src_pinned, int64_t n_words, void *stream)
+{
+    DSKV_REQUIRE(n_words >= 0 && n_words <= (int64_t(1) << 28), "upload_words: %lld words out of range",
+                 (long long)n_words);
+    if (n_words == 0) return 0;
+    DSKV_REQUIRE(dst && src_pinned, "upload_words: null pointer");
+    DSKV_REQUIRE((uintptr_t)dst % 16 == 0 && (uintptr_t)src_pinned % 16 == 0,
+                 "upload_words: both buffers must start on a 16-byte boundary");
+    const long quads = n_words / 4;
+    hipLaunchKernelGGL(dskv::upload_words_kernel, dim3((unsigned)(quads / 256 + 1)), dim3(256), 0,
+                       (hipStream_t)stream, (uint32_t *)dst, (const uint32_t *)src_pinned,
+                       (long)n_words);
+    DSKV_LAUNCH_CHECK("upload_words");
+    return 0;
+}
 
 extern "C" int dskv_gather_pages(void *chunk, const void *pool, const int32_t *page_ids,
                                  int32_t n_pages, int32_t n_layers, int64_t layer_stride_bytes,

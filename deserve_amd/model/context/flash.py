@@ -8,9 +8,9 @@ are exposed and the last page holds (current_len - 1) % P + 1 tokens.
 
 The reference builds six small device tensors with a cat of B device slices and
 five host-to-device constructions per step.  Here all six arrays are laid out in
-ONE pinned host buffer and reach the device in ONE async copy; the device
-tensors of the context are views of that upload, and the host copies are kept
-(``host`` dict) so the attention planner never reads back from the device.
+ONE pinned staging block and reach the device through ONE upload kernel; the
+device tensors of the context are views of that upload, and the host arrays are
+kept (``host`` dict) so the attention planner never reads back from the device.
 """
 from __future__ import annotations
 
@@ -20,6 +20,7 @@ from typing import Dict, List, Sequence
 import numpy as np
 import torch
 
+from deserve_amd import staging
 from deserve_amd.kvcache.paged.kvcache import PagedKVCache
 from deserve_amd.kvcache.paged.page_pool import GpuPagePool
 from deserve_amd.model.context.forward import PagedForwardCtx
@@ -58,34 +59,23 @@ def build_host_metadata(task_datas: Sequence[TaskData],
 
 
 class StagedUpload:
-    """An int32 device buffer that stays where it is from step to step, fed through pinned
-    staging: for callers that replay captured launches (the kernels then find their inputs
-    at the same addresses every step).  The copy to the device is asynchronous, so the
-    staging a step fills must not be the one an earlier, still pending copy reads from:
-    there are two, used in turn, and a staging buffer is handed out again only after the
-    copy that last read it has run."""
+    """An int32 device buffer that stays where it is from step to step, fed from pinned
+    staging blocks: for callers that replay captured launches (the kernels then find their
+    inputs at the same addresses every step)."""
 
     def __init__(self, words: int, device: torch.device) -> None:
         self.dev = torch.empty((words,), dtype=torch.int32, device=device)
-        self._host = [torch.empty((words,), dtype=torch.int32, pin_memory=True) for _ in range(2)]
-        self._copied = [torch.cuda.Event(), torch.cuda.Event()]
-        self._pending = [False, False]
-        self._turn = 0
+        self._block = None
 
     def staging(self) -> torch.Tensor:
-        """The pinned buffer to fill for the next upload (waits for its previous copy)."""
-        self._turn ^= 1
-        if self._pending[self._turn]:
-            self._copied[self._turn].synchronize()
-            self._pending[self._turn] = False
-        return self._host[self._turn]
+        """A pinned buffer to fill for the next upload."""
+        self._block = staging.take(self.dev.numel())
+        return self._block.tensor
 
     def upload(self, words: int) -> None:
-        """Enqueues the copy of the first `words` words of the current staging buffer."""
-        t = self._turn
-        self.dev[:words].copy_(self._host[t][:words], non_blocking=True)
-        self._copied[t].record()
-        self._pending[t] = True
+        """Enqueues the copy of the first `words` words of the staging buffer handed out last."""
+        block, self._block = self._block, None
+        staging.upload(block, self.dev, words)
 
 
 class MetadataBuffers(StagedUpload):
@@ -98,30 +88,32 @@ class MetadataBuffers(StagedUpload):
 
 def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
                     buffers: "MetadataBuffers | None" = None):
-    """One pinned staging buffer, one async copy; returns (device views, host views)."""
+    """One pinned staging block, one upload kernel; returns (device views, host views).
+    The host views are the arrays of `meta` themselves, not the staging block."""
     sizes = [meta[f].shape[0] for f in _FIELDS]
     # each array starts on a 16-byte boundary
     starts, total = [], 0
     for n in sizes:
         starts.append(total)
         total += (n + 3) // 4 * 4
-    use_gpu = torch.device(device).type == "cuda"
-    if buffers is not None:
-        if total > buffers.dev.numel():
+    host_views = {f: torch.from_numpy(meta[f]) for f in _FIELDS}
+    if torch.device(device).type != "cuda":
+        dev = torch.zeros((max(total, 4),), dtype=torch.int32)
+        for f, s, n in zip(_FIELDS, starts, sizes):
+            dev[s: s + n] = host_views[f]
+    else:
+        if buffers is not None and total > buffers.dev.numel():
             raise ValueError(f"step metadata needs {total} words, the buffers hold {buffers.dev.numel()}")
-        staging = buffers.staging()
-    else:
-        staging = torch.empty((max(total, 4),), dtype=torch.int32, pin_memory=use_gpu)
-    host_np = staging.numpy()
-    for f, s, n in zip(_FIELDS, starts, sizes):
-        host_np[s: s + n] = meta[f]
-    if buffers is not None:
-        dev = buffers.dev
-        buffers.upload(total)
-    else:
-        dev = staging.to(device, non_blocking=True) if use_gpu else staging
+        block = None if buffers is not None else staging.take(total)
+        host_np = (buffers.staging() if buffers is not None else block.tensor).numpy()
+        for f, s, n in zip(_FIELDS, starts, sizes):
+            host_np[s: s + n] = meta[f]
+        if buffers is not None:
+            dev = buffers.dev
+            buffers.upload(total)
+        else:
+            dev = staging.to_device(block, total, device)
     dev_views = {f: dev[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
-    host_views = {f: staging[s: s + n] for f, s, n in zip(_FIELDS, starts, sizes)}
     return dev_views, host_views
 
 

@@ -15,7 +15,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from deserve_amd import _lib
+from deserve_amd import _lib, staging
 
 
 def _i32(t: torch.Tensor) -> torch.Tensor:
@@ -133,7 +133,8 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
                 raise ValueError(f"plan buffer holds {plan_buffers.dev.numel()} words, {cap} may be needed")
             plan = plan_buffers.staging()
         else:
-            plan = torch.empty((max(cap, 1),), dtype=torch.int32, pin_memory=True)
+            block = staging.take(max(cap, 1))
+            plan = block.tensor
         n_items, n_wgs = ctypes.c_int32(), ctypes.c_int32()
         words, ws = ctypes.c_int64(), ctypes.c_int64()
         rc = L.dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, page_size,
@@ -144,12 +145,11 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         if ws.value > self._workspace.numel() * self._workspace.element_size():
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
-        self._plan_host = plan                       # keep alive until the upload has run
         if plan_buffers is not None:
             self._plan = plan_buffers.dev
             plan_buffers.upload(max(words.value, 1))
         else:
-            self._plan = plan[: max(words.value, 1)].to(indices.device, non_blocking=True)
+            self._plan = staging.to_device(block, max(words.value, 1), indices.device)
         self._planned = True
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,
@@ -188,14 +188,14 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         nnz = int(h_qo[-1]) if batch > 0 else 0
         L = _lib.lib()
         cap = L.dskv_prefill_plan_bound(batch, nnz)
-        tiles = torch.empty((max(cap, 2),), dtype=torch.int32, pin_memory=True)
+        block = staging.take(max(cap, 2))
+        tiles = block.tensor
         n_tiles = ctypes.c_int32()
         rc = L.dskv_prefill_plan(h_qo.data_ptr(), batch, num_qo_heads, num_kv_heads,
                                  tiles.data_ptr(), cap, ctypes.byref(n_tiles))
         _lib.check(rc, "prefill begin_forward")
         self._batch, self._nnz, self._n_tiles = batch, nnz, n_tiles.value
-        self._tiles_host = tiles
-        self._tiles = tiles[: max(2 * n_tiles.value, 2)].to(paged_kv_indices.device, non_blocking=True)
+        self._tiles = staging.to_device(block, max(2 * n_tiles.value, 2), paged_kv_indices.device)
         self._planned = True
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor, causal: bool = True,

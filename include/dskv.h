@@ -64,6 +64,17 @@ int dskv_scatter_pages(void *pool, const void *chunk, const int32_t *page_ids, i
                        int64_t row_begin, int64_t row_end, void *stream);
 
 /*
+ * Upload of n_words 32-bit words of per-step metadata from pinned host memory
+ * to the device by a kernel on `stream` (no copy engine involved).  Replaces
+ * the host-to-device constructions torch.tensor(..., device=main_device) of
+ * model/context/flash.py:46-64 and the plan upload inside flashinfer's
+ * begin_forward (execution/exec.py:184-192).  src_pinned must be host memory
+ * the device can read (hipHostMalloc / a pinned torch tensor) and must keep its
+ * contents until the kernel has run; both pointers 16-byte aligned.
+ */
+int dskv_upload_words(void *dst, const void *src_pinned, int64_t n_words, void *stream);
+
+/*
  * Paged decode attention.  Replaces BatchDecodeWithPagedKVCacheWrapper
  * begin_forward (execution/exec.py:184-192) = dskv_decode_plan, and
  * forward (model/layer/attention.py:185) = dskv_decode_attn.

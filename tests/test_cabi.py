@@ -50,6 +50,8 @@ def test_argument_errors_return_negative_codes_without_a_gpu():
     assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 2, 0, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
     assert lib.dskv_decode_attn_phases(16, 16, 16, 16, 16, 2, 2, None, 0, 2, 32, 8, 128, 16, 0.1, 2, 0, None) == -1
     assert lib.dskv_apply_rope(16, 16, 16, 16, 16, 16, 1, 1, 32, 8, 130, 5e5, 2, None) == -1
+    assert lib.dskv_upload_words(16, 16, -1, None) == -1 and lib.dskv_upload_words(None, None, 0, None) == 0
+    assert lib.dskv_upload_words(16, 24, 4, None) == -1 and "16-byte" in _lib.last_error()
     assert lib.dskv_swap_slice(16, 64, 128, 2, 16, 16, None, None) == -1             # stride < slice
     assert lib.dskv_swap_slice(None, 0, 0, 0, None, None, None, None) == 0
     assert lib.dskv_swap_wait(None) == -1 and lib.dskv_swap_out_async(None, 1, 1, 1, 1, 1, 64, 64, None) == -1

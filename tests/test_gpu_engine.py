@@ -300,3 +300,38 @@ def test_graphed_decode_step_matches_eager_steps():
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16))
     assert step.captures == 2
+
+
+@pytest.mark.gpu
+def test_staged_uploads_are_exact_and_blocks_wait_for_their_readers():
+    """dskv_upload_words through the staging pool: every length (quads + tail words), and a
+    host that refills blocks while earlier uploads are still queued behind a long kernel."""
+    from deserve_amd import staging
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(5)
+    for words in (1, 3, 4, 5, 255, 1023, 1024, 1025, 100_001):
+        src = rng.integers(-2**31, 2**31 - 1, size=words, dtype=np.int64).astype(np.int32)
+        blk = staging.take(words)
+        blk.tensor.numpy()[:words] = src
+        dst = torch.full((words + 8,), 77, dtype=torch.int32, device=dev)
+        staging.upload(blk, dst, words)
+        got = dst.cpu().numpy()
+        assert np.array_equal(got[:words], src) and np.all(got[words:] == 77), words
+    # queue a long kernel, then 32 uploads whose blocks the host fills back to back
+    busy = torch.empty((1 << 28,), dtype=torch.int32, device=dev)
+    busy.zero_()
+    outs, refs = [], []
+    for i in range(32):
+        src = rng.integers(0, 1 << 30, size=5000, dtype=np.int64).astype(np.int32)
+        blk = staging.take(5000)
+        blk.tensor.numpy()[:5000] = src
+        outs.append(staging.to_device(blk, 5000, dev))
+        refs.append(src)
+        if i % 8 == 0:
+            busy.add_(1)
+    torch.cuda.synchronize()
+    for o, r in zip(outs, refs):
+        assert np.array_equal(o.cpu().numpy(), r)
+    with pytest.raises(ValueError):
+        staging.upload(staging.take(4), torch.zeros(2, dtype=torch.int32, device=dev), 4)
