@@ -63,21 +63,41 @@ static int wait_all(dskv_swap *h)
     return 0;
 }
 
-// Copy the caller's page ids into the arena and start their upload on `s`.
+// Copy the caller's page ids into the arena and start their upload on `s`: a kernel
+// reading the pinned mirror (slots are multiples of four words, as it wants), so the
+// copy engines carry page data only.
 static int stage_ids(dskv_swap *h, const int32_t *ids, int32_t n, hipStream_t s, int32_t **dev_out)
 {
-    DSKV_REQUIRE(n <= h->ids_capacity, "swap: %d page ids exceed the engine's limit of %lld", n,
+    const int64_t slot = ((int64_t)n + 3) / 4 * 4;
+    DSKV_REQUIRE(slot <= h->ids_capacity, "swap: %d page ids exceed the engine's limit of %lld", n,
                  (long long)h->ids_capacity);
-    if (h->ids_used + n > h->ids_capacity) {
+    if (h->ids_used + slot > h->ids_capacity) {
         int rc = wait_all(h);   // arena full: drain, then start over
         if (rc) return rc;
     }
     int32_t *host = h->ids_host + h->ids_used;
     int32_t *dev = h->ids_dev + h->ids_used;
     std::copy(ids, ids + n, host);
-    h->ids_used += n;
-    DSKV_HIP(hipMemcpyAsync(dev, host, (size_t)n * sizeof(int32_t), hipMemcpyHostToDevice, s));
+    h->ids_used += slot;
+    int rc = dskv_upload_words(dev, host, n, s);
+    if (rc) return rc;
     *dev_out = dev;
+    return 0;
+}
+
+// The gather and scatter kernels index the pool by page id: ids outside a layer are
+// refused here, on the host.
+static int check_ids(const char *who, const int32_t *ids, int32_t n, int64_t layer_stride_bytes,
+                     int64_t page_bytes)
+{
+    int32_t top = 0;
+    for (int32_t i = 0; i < n; i++) {
+        DSKV_REQUIRE(ids[i] >= 0, "%s: negative page id %d at %d", who, ids[i], i);
+        top = std::max(top, ids[i]);
+    }
+    DSKV_REQUIRE(((int64_t)top + 1) * page_bytes <= layer_stride_bytes,
+                 "%s: page id %d lies outside a layer of %lld bytes", who, top,
+                 (long long)layer_stride_bytes);
     return 0;
 }
 
@@ -205,6 +225,7 @@ extern "C" int dskv_swap_out_async(dskv_swap_t *h, void *host_dst, const void *p
     const int64_t rows = (int64_t)n_pages * n_layers;
     if (rows == 0) return 0;
     DSKV_REQUIRE(host_dst && pool && page_ids_host, "swap_out: null pointer argument");
+    if ((rc = check_ids("swap_out", page_ids_host, n_pages, layer_stride_bytes, page_bytes))) return rc;
     const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
     DSKV_REQUIRE(rows_per_chunk >= 1, "swap_out: a page (%lld bytes) does not fit the staging buffer",
                  (long long)page_bytes);
@@ -235,6 +256,7 @@ extern "C" int dskv_swap_in_async(dskv_swap_t *h, void *pool, const void *host_s
     const int64_t rows = (int64_t)n_pages * n_layers;
     if (rows == 0) return 0;
     DSKV_REQUIRE(host_src && pool && page_ids_host, "swap_in: null pointer argument");
+    if ((rc = check_ids("swap_in", page_ids_host, n_pages, layer_stride_bytes, page_bytes))) return rc;
     const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
     DSKV_REQUIRE(rows_per_chunk >= 1, "swap_in: a page (%lld bytes) does not fit the staging buffer",
                  (long long)page_bytes);
@@ -266,6 +288,8 @@ extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const vo
     if (rows == 0) return 0;
     DSKV_REQUIRE(host_dst && host_src && pool && page_ids_host,
                  "swap_exchange: null pointer argument");
+    if ((rc = check_ids("swap_exchange", page_ids_host, n_pages, layer_stride_bytes, page_bytes)))
+        return rc;
     const int64_t rows_per_chunk = h->staging_bytes / page_bytes;
     DSKV_REQUIRE(rows_per_chunk >= 1,
                  "swap_exchange: a page (%lld bytes) does not fit the staging buffer",

@@ -189,8 +189,8 @@ int dskv_swap_slice(void *slice_base, int64_t layer_stride_bytes, int64_t slice_
  * per-task copies KVCacheManager.copy_gpu_to_cpu / copy_cpu_to_gpu
  * (kvcache/manager.py:24-86); host layout (n_layers*n_pages, page_bytes), layer
  * major then page_ids order.  page_ids is a HOST int32 array (copied at call
- * time).  after_stream: work already enqueued there is waited for before the
- * pool is touched.  dskv_swap_wait blocks the host until everything enqueued
+ * time); ids outside a layer are refused with DSKV_E_INVAL.  after_stream:
+ * work already enqueued there is waited for before the pool is touched.  dskv_swap_wait blocks the host until everything enqueued
  * on the handle is done; dskv_swap_fence makes `stream` wait for it instead.
  */
 typedef struct dskv_swap dskv_swap_t;

@@ -111,6 +111,34 @@ def test_swap_engine_scattered_pages_round_trip(staging_mib, n):
     eng.close()
 
 
+def test_swap_engine_refuses_page_ids_outside_the_pool():
+    """The gather and scatter kernels index the pool by page id; a bad id is refused on the
+    host, before anything is launched, and the engine keeps working."""
+    from deserve_amd.kvcache import _native
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.pinned.pinned_memory import pinned_empty
+
+    _announce("swap engine refusals")
+    L, P, num_pages = 2, 16, 8
+    pool = GpuPagePool(L, num_pages, P, DEV, torch.bfloat16)
+    before = _fill_random(pool.pages, 7)
+    eng = _native.SwapEngine(1 << 20)
+    host = pinned_empty((L * 2,) + tuple(pool.pages.shape[2:]), torch.bfloat16)
+    with pytest.raises(ValueError, match="page id"):
+        eng.swap_out(host, pool, torch.tensor([1, num_pages], dtype=torch.int32))
+    with pytest.raises(ValueError, match="page id"):
+        eng.swap_in(pool, host, torch.tensor([-1, 2], dtype=torch.int32))
+    with pytest.raises(ValueError, match="page id"):
+        eng.exchange(host, host.clone().pin_memory(), pool, torch.tensor([0, 1 << 30], dtype=torch.int32))
+    eng.wait()
+    assert _same_bits(_bits(pool.pages), before)
+    ids = torch.tensor([1, 5], dtype=torch.int32)
+    eng.swap_out(host, pool, ids)
+    eng.wait()
+    assert _same_bits(_bits(host), orc.gather_pages(before, ids.numpy()))
+    eng.close()
+
+
 def test_manager_offload_reload_keeps_bits_and_reference_call_order():
     from deserve_amd.kvcache.manager import KVCacheManager
     from deserve_amd.kvcache.paged.chunk_pool import CpuChunkPool
