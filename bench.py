@@ -258,7 +258,9 @@ def prefill_section(seed: int):
     w.begin_forward(qo_indptr=c.indptr, paged_kv_indptr=c.kv_page_indptr,
                     paged_kv_indices=c.kv_page_indices, paged_kv_last_page_len=c.kv_last_page_lens,
                     num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
-                    qo_indptr_host=c.host["indptr"])
+                    qo_indptr_host=c.host["indptr"],
+                    paged_kv_indptr_host=c.host["kv_page_indptr"],
+                    paged_kv_last_page_len_host=c.host["kv_last_page_lens"])
     flops = 4 * Hq * D * sum(n * int(p) + n * (n + 1) // 2 for p in prior)
 
     def median_us(fn, reps=5):

@@ -22,6 +22,8 @@
 // so (with 8 kv heads) all query tiles of one kv head share one XCD's L2.
 #include "kv_tile.h"
 
+#include <vector>
+
 #include <algorithm>
 
 namespace dskv {
@@ -513,9 +515,10 @@ extern "C" int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz)
     return 2 * ((int64_t)batch + nnz);
 }
 
-extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, int32_t batch, int32_t n_qo_heads,
-                                 int32_t n_kv_heads, int32_t *tile_info_host,
-                                 int64_t capacity_words, int32_t *n_tiles_out)
+extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
+                                 int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads,
+                                 int32_t *tile_info_host, int64_t capacity_words,
+                                 int32_t *n_tiles_out)
 {
     using namespace dskv;
     DSKV_REQUIRE(batch >= 0 && n_tiles_out, "prefill_plan: bad arguments");
@@ -527,8 +530,7 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, int32_t batch, i
     DSKV_REQUIRE(qo_indptr_host && tile_info_host, "prefill_plan: null pointer argument");
     const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads);
     int64_t n = 0;
-    // later query tiles of a request see more keys: emit them first so the
-    // longest workgroups start first
+    // later query tiles of a request see more keys: emit them first
     for (int b = 0; b < batch; b++) {
         const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
         DSKV_REQUIRE(n_b >= 0, "prefill_plan: qo_indptr not monotone at %d", b);
@@ -545,6 +547,25 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, int32_t batch, i
     }
     DSKV_REQUIRE(n < (int64_t(1) << 31), "prefill_plan: too many tiles");
     *n_tiles_out = (int32_t)n;
+    if (kv_len_host && n > 1) {
+        // Workgroups are dispatched in tile order and a tile's time grows with the keys its
+        // last row sees: longest first, so the short ones fill the end of the launch
+        // (request order left a fifth of the wave slots idle on mixed lengths).
+        struct Tile { int32_t b, row; int64_t keys; };
+        std::vector<Tile> order((size_t)n);
+        for (int64_t i = 0; i < n; i++) {
+            const int32_t b = tile_info_host[2 * i], row = tile_info_host[2 * i + 1];
+            const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
+            const int64_t last_row = std::min<int64_t>(row + rows, n_b) - 1;
+            order[(size_t)i] = {b, row, std::max<int64_t>((int64_t)kv_len_host[b] - n_b + last_row + 1, 0)};
+        }
+        std::stable_sort(order.begin(), order.end(),
+                         [](const Tile &x, const Tile &y) { return x.keys > y.keys; });
+        for (int64_t i = 0; i < n; i++) {
+            tile_info_host[2 * i] = order[(size_t)i].b;
+            tile_info_host[2 * i + 1] = order[(size_t)i].row;
+        }
+    }
     return 0;
 }
 

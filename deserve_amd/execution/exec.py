@@ -127,7 +127,10 @@ class BatchPrefill(BatchExec):
             wrapper.begin_forward(qo_indptr=ctx.indptr, paged_kv_indptr=ctx.kv_page_indptr,
                                   paged_kv_indices=ctx.kv_page_indices,
                                   paged_kv_last_page_len=ctx.kv_last_page_lens,
-                                  qo_indptr_host=ctx.host["indptr"], **self._shape_kwargs())
+                                  qo_indptr_host=ctx.host["indptr"],
+                                  paged_kv_indptr_host=ctx.host["kv_page_indptr"],
+                                  paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"],
+                                  **self._shape_kwargs())
             self.prefill_ctx = ctx
 
     def step(self, ignore_eos: bool) -> BatchResult:

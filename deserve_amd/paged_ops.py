@@ -179,7 +179,11 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
     def begin_forward(self, qo_indptr: torch.Tensor, paged_kv_indptr: torch.Tensor,
                       paged_kv_indices: torch.Tensor, paged_kv_last_page_len: torch.Tensor,
                       num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int, *,
-                      qo_indptr_host: Optional[torch.Tensor] = None, **_ignored) -> None:
+                      qo_indptr_host: Optional[torch.Tensor] = None,
+                      paged_kv_indptr_host: Optional[torch.Tensor] = None,
+                      paged_kv_last_page_len_host: Optional[torch.Tensor] = None, **_ignored) -> None:
+        """The *_host arguments are host copies of the index tensors (the planner runs on the
+        host; without them it reads the device tensors back, which synchronises)."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
@@ -191,7 +195,12 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         block = staging.take(max(cap, 2))
         tiles = block.tensor
         n_tiles = ctypes.c_int32()
-        rc = L.dskv_prefill_plan(h_qo.data_ptr(), batch, num_qo_heads, num_kv_heads,
+        # kv lengths order the tiles longest first
+        h_indptr = self._host(paged_kv_indptr, paged_kv_indptr_host).to(torch.int64)
+        h_last = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host).to(torch.int64)
+        n_pages = h_indptr[1:] - h_indptr[:-1]
+        kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
+        rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,
                                  tiles.data_ptr(), cap, ctypes.byref(n_tiles))
         _lib.check(rc, "prefill begin_forward")
         self._batch, self._nnz, self._n_tiles = batch, nnz, n_tiles.value

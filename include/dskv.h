@@ -132,11 +132,14 @@ int dskv_decode_attn_phases(void *out, const void *q, const void *pages_layer,
  * (request, first query row of the tile within the request) built by
  * dskv_prefill_plan from the host copy of qo_indptr (needs at most
  * dskv_prefill_plan_bound(batch, nnz) words); unused (may be NULL) for fp32.
+ * kv_len_host (batch host int32, may be NULL): the requests' kv lengths; with
+ * them the tiles are ordered longest first, which balances a launch over
+ * requests of mixed lengths (the result does not depend on the order).
  */
 int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz);
-int dskv_prefill_plan(const int32_t *qo_indptr_host, int32_t batch, int32_t n_qo_heads,
-                      int32_t n_kv_heads, int32_t *tile_info_host, int64_t capacity_words,
-                      int32_t *n_tiles_out);
+int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host, int32_t batch,
+                      int32_t n_qo_heads, int32_t n_kv_heads, int32_t *tile_info_host,
+                      int64_t capacity_words, int32_t *n_tiles_out);
 int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const void *pages_layer,
                       const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
                       const int32_t *kv_last_page_len, const int32_t *tile_info_dev,

@@ -140,7 +140,7 @@ def test_prefill_plan_tiles_cover_all_query_rows():
         cap = lib.dskv_prefill_plan_bound(4, 520)
         tiles = np.zeros(cap, np.int32)
         n = ctypes.c_int32()
-        assert lib.dskv_prefill_plan(qo.ctypes.data, 4, hq, hkv, tiles.ctypes.data, cap, ctypes.byref(n)) == 0
+        assert lib.dskv_prefill_plan(qo.ctypes.data, None, 4, hq, hkv, tiles.ctypes.data, cap, ctypes.byref(n)) == 0
         t = tiles[: 2 * n.value].reshape(-1, 2)
         group = hq // hkv
         rows = None
@@ -156,4 +156,25 @@ def test_prefill_plan_tiles_cover_all_query_rows():
                 assert rows % max(32 // group, 1) == 0 if group <= 32 else rows == 1
             assert starts == list(range(0, nb, rows))
     n = ctypes.c_int32()
-    assert lib.dskv_prefill_plan(qo.ctypes.data, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2
+    assert lib.dskv_prefill_plan(qo.ctypes.data, None, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2
+
+
+def test_prefill_plan_with_kv_lengths_orders_tiles_longest_first():
+    """Same tiles as without lengths, ordered by the keys their last row sees (descending)."""
+    lib = _lib.lib()
+    qo = np.array([0, 512, 512, 519, 520, 1000], np.int32)
+    kv_len = np.array([600, 0, 4000, 1, 480], np.int32)
+    cap = lib.dskv_prefill_plan_bound(5, 1000)
+    plain, ordered = np.zeros(cap, np.int32), np.zeros(cap, np.int32)
+    n0, n1 = ctypes.c_int32(), ctypes.c_int32()
+    assert lib.dskv_prefill_plan(qo.ctypes.data, None, 5, 32, 8, plain.ctypes.data, cap, ctypes.byref(n0)) == 0
+    assert lib.dskv_prefill_plan(qo.ctypes.data, kv_len.ctypes.data, 5, 32, 8, ordered.ctypes.data, cap,
+                                 ctypes.byref(n1)) == 0
+    assert n0.value == n1.value
+    a = plain[: 2 * n0.value].reshape(-1, 2)
+    b = ordered[: 2 * n1.value].reshape(-1, 2)
+    assert sorted(map(tuple, a.tolist())) == sorted(map(tuple, b.tolist()))
+    rows = 64                                             # 8 waves x 32 // 4 query rows
+    n_b = np.diff(qo)
+    keys = [kv_len[r] - n_b[r] + min(s + rows, n_b[r]) for r, s in b]
+    assert keys == sorted(keys, reverse=True) and keys[0] == 4000

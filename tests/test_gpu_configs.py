@@ -194,7 +194,9 @@ def test_config4_chunked_prefill_full_batch_two_layers():
     w.begin_forward(qo_indptr=ctx.indptr, paged_kv_indptr=ctx.kv_page_indptr,
                     paged_kv_indices=ctx.kv_page_indices, paged_kv_last_page_len=ctx.kv_last_page_lens,
                     num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
-                    qo_indptr_host=ctx.host["indptr"])
+                    qo_indptr_host=ctx.host["indptr"],
+                    paged_kv_indptr_host=ctx.host["kv_page_indptr"],
+                    paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"])
     before = [_checksum(pool.pages[l]) for l in range(L)]
     indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
     # slots the chunk will overwrite: positions prior_b .. prior_b + n - 1
