@@ -58,7 +58,10 @@ constexpr float kRescaleSlack = 8.f;
 //   A operand: row r, k = 8h .. 8h+7.   B operand: column r, k = 8h .. 8h+7.
 //   C/D: column r, rows 8i + 4h + j in register 4i + j (i, j = 0..3).
 template <int DT, bool kRowsSharePage>
-__global__ __launch_bounds__(64 * kPrefillWaves) void prefill_attn_mfma_kernel(
+#ifndef DSKV_PREFILL_MIN_WAVES
+#define DSKV_PREFILL_MIN_WAVES 1
+#endif
+__global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void prefill_attn_mfma_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
     const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
     const int32_t *__restrict__ kv_indices, const int32_t *__restrict__ kv_indptr,
