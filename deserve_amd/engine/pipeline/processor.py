@@ -27,7 +27,8 @@ from deserve_amd.task import SamplingParams, TaskData, TaskManager
 
 @dataclass
 class StepRequest:
-    """Data of deserve_worker/request.py:137-146 (the wire encoding is not part of the path)."""
+    """Data of deserve_worker/request.py:137-146; into_safetensors / from_safetensors are the
+    pair that deserve_amd.serde.dumps / loads put on the wire (request.py:199-210)."""
     microbatch_id: int
     xs: object
     exec_task_ids: List[str] = field(default_factory=list)
@@ -59,6 +60,29 @@ class StepRequest:
 
     def get_bsz(self) -> int:
         return len(self.exec_task_ids)
+
+    def into_safetensors(self):
+        return {"xs": self.xs}, {
+            "group_id": self.microbatch_id,
+            "exec_task_ids": self.exec_task_ids,
+            "exec_seqlens": self.exec_seqlens,
+            "cancel_task_ids": self.cancel_task_ids,
+            "offload_task_ids": self.offload_task_ids,
+            "reload_task_ids": self.reload_task_ids,
+            "init_tasks": self.init_tasks,
+        }
+
+    @staticmethod
+    def from_safetensors(tensors, metadata, device=None) -> "StepRequest":
+        """Inverse of into_safetensors; xs is moved to `device` if one is given."""
+        xs = tensors["xs"] if device is None else tensors["xs"].to(device)
+        return StepRequest(metadata["group_id"], xs, list(metadata["exec_task_ids"]),
+                           list(metadata["exec_seqlens"]), list(metadata["cancel_task_ids"]),
+                           list(metadata["offload_task_ids"]), list(metadata["reload_task_ids"]),
+                           dict(metadata["init_tasks"]))
+
+    def get_tensors_size(self) -> int:
+        return self.xs.numel() * self.xs.element_size()
 
     def refresh(self) -> None:
         """A request that comes round again carries only decodes (request.py:193-197)."""

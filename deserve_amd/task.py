@@ -20,6 +20,17 @@ class SamplingParams:
     max_new_tokens: int = 4096
     dump_probs_num: int = 0
 
+    def model_dump(self) -> dict:
+        """The fields as a dict (the reference's pydantic model offers the same call)."""
+        return dict(self.__dict__)
+
+    def __setstate__(self, state) -> None:
+        # a pickle of the reference's pydantic model carries its fields under "__dict__"
+        fields = state.get("__dict__", state) if isinstance(state, dict) else state
+        for name in ("temperature", "top_p", "max_seq_len", "max_new_tokens", "dump_probs_num"):
+            if name in fields:
+                setattr(self, name, fields[name])
+
 
 @dataclass
 class TaskData:
