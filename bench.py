@@ -43,6 +43,11 @@ def parse_args():
     ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill section")
     ap.add_argument("--no-fragmented", action="store_true", help="skip the fragmented long-context section")
+    ap.add_argument("--no-fused-append", action="store_true",
+                    help="append with a launch of its own instead of inside the attention launch")
+    ap.add_argument("--steps-in-flight", type=int, default=2,
+                    help="steps the host may have queued on the GPU (a stage hands every step's "
+                         "output on before it starts the next but one); 0 = no limit")
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--section", choices=["swap", "fragmented"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
@@ -481,8 +486,11 @@ def main() -> int:
     step_bytes = []
     attn_bytes_layer = []
 
+    fused = not a.no_fused_append and not a.rope
+
     def one_step(timed: bool):
-        """prepare (metadata + plan, one upload each) then L x (append, attention)."""
+        """prepare (metadata + plan, one upload each) then L x (append + attention: one launch
+        for both, or two with --no-fused-append)."""
         c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, decode_wrapper)
         decode_wrapper.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
                                      last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
@@ -495,18 +503,22 @@ def main() -> int:
             if a.rope:
                 q, k = apply_rope(q, k, c.indptr, c.offsets, interleave=True, rope_theta=5e5)
             pages = wl.pool.get_layered_pages(layer)
-            append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
-                                  c.kv_last_page_lens)
+            if fused:
+                new_kv = dict(k_append=k, v_append=v)    # the attention launch writes the token
+            else:
+                new_kv = {}
+                append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
+                                      c.kv_last_page_lens)
             launch_no[0] += 1
             if timed and not a.no_kernel_events and launch_no[0] % max(a.event_every, 1) == 0:
                 s, t = ev_pool[len(ev_pairs)]
                 s.record()
-                out = decode_wrapper.forward(q, pages, phases=1)
+                out = decode_wrapper.forward(q, pages, phases=1, **new_kv)
                 t.record()
                 decode_wrapper.forward(q, pages, phases=2, out=out)
                 ev_pairs.append((s, t))
             else:
-                decode_wrapper.forward(q, pages)
+                decode_wrapper.forward(q, pages, **new_kv)
         decode_wrapper.end_forward()
         if timed:
             kv_lens = np.array([t.start_pos + 1 for t in wl.tasks], dtype=np.int64)
@@ -522,9 +534,23 @@ def main() -> int:
     for _ in range(a.warmup):
         last_ctx = one_step(False)
     torch.cuda.synchronize()
+    in_flight = [torch.cuda.Event() for _ in range(max(a.steps_in_flight, 0))]
+
+    def wait_turn(i: int):
+        """Blocks until step i - len(in_flight) has run; returns the event to record after step i."""
+        if not in_flight:
+            return None
+        ev = in_flight[i % len(in_flight)]
+        if i >= len(in_flight):
+            ev.synchronize()
+        return ev
+
     t0 = time.perf_counter()
-    for _ in range(a.steps):
+    for i in range(a.steps):
+        ev = wait_turn(i)
         last_ctx = one_step(True)
+        if ev is not None:
+            ev.record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
@@ -540,7 +566,8 @@ def main() -> int:
                                "step = host plan + 16 x (append 1 token + paged decode attention)"
                                + (" + RoPE" if a.rope else ""),
                    "batch": wl.batch, "layers": L, "kv_tokens": int(sum(t.start_pos for t in wl.tasks)),
-                   "work_items": decode_wrapper._n_items, "workgroups": decode_wrapper._n_workgroups, "seed": a.seed},
+                   "work_items": decode_wrapper._n_items, "workgroups": decode_wrapper._n_workgroups, "seed": a.seed,
+                   "append": "inside the attention launch" if fused else "own launch"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "stage_tokens_per_s": round(wl.batch / (elapsed / a.steps), 1),
     }
@@ -555,7 +582,7 @@ def main() -> int:
         tfile = os.path.join(ROOT, "profiles", "decode_attn_cfg2_traffic.json")
         if os.path.exists(tfile):
             traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
-        out["roofline"] = {"bound": "hbm", "kernel": "decode_attn_mfma_kernel<bf16> (split-KV pass)",
+        out["roofline"] = {"bound": "hbm", "kernel": "decode_attn_mfma_kernel<bf16> (split-KV pass" + (", writes the step's token first)" if fused else ")"),
                            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                            "avg_launch_us": round(avg_ms * 1e3, 2), "launches": len(times_ms),
@@ -580,8 +607,11 @@ def main() -> int:
             graphed()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(graph_steps - 4):
+        for i in range(graph_steps - 4):
+            ev = wait_turn(i)
             graphed()
+            if ev is not None:
+                ev.record()
         torch.cuda.synchronize()
         g_ms = (time.perf_counter() - t0) / (graph_steps - 4) * 1e3
         out["graph"] = {"ms_per_step": round(g_ms, 4),

@@ -55,7 +55,8 @@ constexpr int kMinTilesPerWorkgroup = 4;
 struct Item {
     int32_t b, tok_begin, tok_end, slot;
     int32_t page_begin;   // kv_page_indptr[b]: start of the request's block table
-    int32_t reserved[3];
+    int32_t tail;         // 1: tok_end is the request's length (the item holds its newest token)
+    int32_t reserved[2];
 };
 static_assert(sizeof(Item) == kItemWords * 4, "plan item layout");
 
@@ -78,10 +79,11 @@ struct LoadCursor {
 #endif
 template <int DT, bool kPageCoversTile>
 __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_attn_mfma_kernel(
-    uint16_t *__restrict__ out, const uint16_t *__restrict__ q, const char *__restrict__ pages,
+    uint16_t *__restrict__ out, const uint16_t *__restrict__ q, const char *pages,
     const int32_t *__restrict__ kv_indices, const Item *__restrict__ items,
     const int32_t *__restrict__ wg_ptr, float *__restrict__ part_o, float *__restrict__ part_ml,
-    int max_slots, int n_qo_heads, int n_kv_heads, int page_shift, float scale_log2)
+    int max_slots, int n_qo_heads, int n_kv_heads, int page_shift, float scale_log2,
+    const uint16_t *__restrict__ k_new, const uint16_t *__restrict__ v_new)
 {
     typedef Elt<DT> E;
     __shared__ __align__(16) char v_lds[kMaxWaves][kVTileBytes];
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     const const_i32_ptr item_words = as_const(reinterpret_cast<const int32_t *>(items));
     auto load_item = [&](int idx) {
         const const_i32_ptr w = item_words + (long)idx * kItemWords;
-        return Item{w[0], w[1], w[2], w[3], w[4], {0, 0, 0}};
+        return Item{w[0], w[1], w[2], w[3], w[4], w[5], {0, 0}};
     };
     const const_i32_ptr indices_c = as_const(kv_indices);
     const int item_begin = as_const(wg_ptr)[blockIdx.x];
@@ -113,6 +115,29 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     kv.page_bytes = 2L * kv.half_bytes;
     kv.head_off = kvh * (kHeadDim * 2);
     char *lds = v_lds[wave];
+
+    // Fused append (k_new != null): the newest token of a request has not been written
+    // to its page yet.  The wave that will read it - kv head `kvh` of the item that ends
+    // the request - writes its 256 bytes of K and of V first and waits until the cache
+    // has them; nobody else reads that row in this launch.
+    if (k_new) {
+        for (int idx = item_begin; idx < item_end; idx++) {
+            const Item it = load_item(idx);
+            if (!it.tail) continue;
+            const int tok = it.tok_end - 1;
+            const long page = indices_c[it.page_begin + (tok >> page_shift)];
+            char *row = const_cast<char *>(pages) + page * kv.page_bytes +
+                        (long)(tok & ((1 << page_shift) - 1)) * kv.row_bytes + kv.head_off;
+            const long src = ((long)it.b * n_kv_heads + kvh) * kHeadDim;
+            if (lane < 16)
+                *reinterpret_cast<u32x4 *>(row + lane * 16) =
+                    *reinterpret_cast<const u32x4 *>(k_new + src + lane * 8);
+            else if (lane < 32)
+                *reinterpret_cast<u32x4 *>(row + kv.half_bytes + (lane - 16) * 16) =
+                    *reinterpret_cast<const u32x4 *>(v_new + src + (lane - 16) * 8);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
 
     // Q rows of one item as the B operand of the score MFMAs (zero beyond the group).
     auto load_q = [&](int item_idx, u32x4 (&dst)[4]) {
@@ -486,7 +511,7 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
     auto share_end = [&](int64_t wg) { return (wg + 1) * total_tiles / wgs; };
     for (int b = 0; b < batch; b++) {
         if (tiles[b] == 0) {
-            items.push_back(Item{b, 0, 0, -1, kv_page_indptr_host[b], {0, 0, 0}});
+            items.push_back(Item{b, 0, 0, -1, kv_page_indptr_host[b], 0, {0, 0}});
             continue;
         }
         const size_t first_item = items.size();
@@ -500,7 +525,7 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
             const int64_t take = std::min(room, tiles[b] - done);
             items.push_back(Item{b, (int32_t)(done * kTile),
                                  (int32_t)std::min<int64_t>((done + take) * kTile, len[b]), -1,
-                                 kv_page_indptr_host[b], {0, 0, 0}});
+                                 kv_page_indptr_host[b], done + take == tiles[b], {0, 0}});
             done += take;
             g0 += take;
         }
@@ -540,14 +565,18 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
     return 0;
 }
 
-extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pages_layer,
-                                       const int32_t *kv_page_indices, const int32_t *plan_dev,
-                                       int32_t n_items, int32_t n_workgroups, void *workspace,
-                                       int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
-                                       int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
-                                       float sm_scale, int32_t dtype, int32_t phases, void *stream)
+namespace dskv {
+
+// k_new / v_new non-null: the fused form, which also writes the step's token of every
+// request into its page slot (MFMA path only).
+static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
+                            const int32_t *kv_page_indices, const int32_t *plan_dev,
+                            int32_t n_items, int32_t n_workgroups, void *workspace,
+                            int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
+                            int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
+                            float sm_scale, int32_t dtype, int32_t phases, void *stream,
+                            const void *k_new, const void *v_new)
 {
-    using namespace dskv;
     DSKV_REQUIRE(phases >= 1 && phases <= 3, "decode_attn: phases must be 1, 2 or 3");
     DSKV_REQUIRE(batch >= 0 && n_items >= 0 && n_workgroups >= 0,
                  "decode_attn: negative batch/n_items/n_workgroups");
@@ -586,6 +615,9 @@ extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pag
     const float scale_log2 = sm_scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
 
+    DSKV_REQUIRE(!k_new || (mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads) && (phases & 1)),
+                 "decode_append_attn: shape or dtype outside the fused kernel (see "
+                 "dskv_decode_append_attn_supported); append and attend separately");
     if (!(phases & 1)) {
         // merge only: the split-KV pass of this plan has already been enqueued
     } else if (mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads)) {
@@ -603,7 +635,7 @@ extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pag
     hipLaunchKernelGGL((decode_attn_mfma_kernel<DT, COVER>), grid, block, 0, s, (uint16_t *)out, \
                        (const uint16_t *)q, (const char *)pages_layer, kv_page_indices, items,   \
                        wg_ptr, part_o, part_ml, (int)max_slots, n_qo_heads, n_kv_heads, shift,   \
-                       scale_log2)
+                       scale_log2, (const uint16_t *)k_new, (const uint16_t *)v_new)
         if (dtype == DSKV_BF16) {
             if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_BF16, true);
             else DSKV_LAUNCH_MFMA(DSKV_BF16, false);
@@ -639,6 +671,49 @@ extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pag
         DSKV_LAUNCH_CHECK("decode_merge_kernel");
     }
     return 0;
+}
+
+}  // namespace dskv
+
+extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pages_layer,
+                                       const int32_t *kv_page_indices, const int32_t *plan_dev,
+                                       int32_t n_items, int32_t n_workgroups, void *workspace,
+                                       int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
+                                       int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
+                                       float sm_scale, int32_t dtype, int32_t phases, void *stream)
+{
+    return dskv::decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items,
+                                  n_workgroups, workspace, workspace_bytes, batch, n_qo_heads,
+                                  n_kv_heads, head_dim, page_size, sm_scale, dtype, phases, stream,
+                                  nullptr, nullptr);
+}
+
+extern "C" int dskv_decode_append_attn_supported(int32_t n_qo_heads, int32_t n_kv_heads,
+                                                 int32_t head_dim, int32_t page_size, int32_t dtype)
+{
+    using namespace dskv;
+    return n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0 && page_size > 0 &&
+           is_pow2(page_size) && mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads);
+}
+
+extern "C" int dskv_decode_append_attn(void *out, const void *q, const void *k_new,
+                                       const void *v_new, void *pages_layer,
+                                       const int32_t *kv_page_indices, const int32_t *plan_dev,
+                                       int32_t n_items, int32_t n_workgroups, void *workspace,
+                                       int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
+                                       int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
+                                       float sm_scale, int32_t dtype, int32_t phases, void *stream)
+{
+    using namespace dskv;
+    if (batch == 0 || n_items == 0) return 0;
+    DSKV_REQUIRE(phases == 1 || phases == 3,
+                 "decode_append_attn: the append belongs to the attention pass (phases 1 or 3)");
+    DSKV_REQUIRE(k_new && v_new, "decode_append_attn: null k_new / v_new");
+    DSKV_REQUIRE(((uintptr_t)k_new | (uintptr_t)v_new) % 16 == 0,
+                 "decode_append_attn: k_new / v_new must be 16-byte aligned");
+    return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
+                            workspace, workspace_bytes, batch, n_qo_heads, n_kv_heads, head_dim,
+                            page_size, sm_scale, dtype, phases, stream, k_new, v_new);
 }
 
 extern "C" int dskv_decode_attn(void *out, const void *q, const void *pages_layer,

@@ -14,11 +14,13 @@ from deserve_amd.paged_ops import (append_paged_kv_cache, apply_rope,
 
 class PagedAttentionCore:
     def __init__(self, n_heads: int, n_kv_heads: int, head_dim: int, rope_theta: float = 500000.0,
-                 use_rope: bool = True, fuse_rope_append: bool = True) -> None:
+                 use_rope: bool = True, fuse_rope_append: bool = True,
+                 fuse_decode_append: bool = True) -> None:
         self.n_local_heads, self.n_local_kv_heads = n_heads, n_kv_heads
         self.head_dim, self.dim = head_dim, n_heads * head_dim
         self.rope_theta, self.use_rope = rope_theta, use_rope
         self.fuse_rope_append = fuse_rope_append
+        self.fuse_decode_append = fuse_decode_append
 
     @torch.inference_mode()
     def paged_forward(self, xq: torch.Tensor, xk: torch.Tensor, xv: torch.Tensor,
@@ -27,6 +29,11 @@ class PagedAttentionCore:
         xk = xk.view(-1, self.n_local_kv_heads, self.head_dim)
         xv = xv.view(-1, self.n_local_kv_heads, self.head_dim)
         pages = ctx.page_pool.get_layered_pages(ctx.layer_id)
+        if (not self.use_rope and isinstance(ctx, FlashDecodeCtx) and self.fuse_decode_append
+                and xk.shape[0] == ctx.bsz and ctx.decode_wrapper.fused_append_supported(xq.dtype)):
+            # a decode step without rotation: the attention launch writes the new token itself
+            out = ctx.decode_wrapper.forward(xq, pages, k_append=xk, v_append=xv)
+            return out.view(-1, self.dim)
         if self.use_rope and self.fuse_rope_append:
             # one kernel: rotated q comes back, rotated k and v go straight into their slots
             xq = rope_append_paged_kv_cache(xq, xk, xv, ctx.indptr, ctx.offsets, pages,

@@ -152,10 +152,22 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
             self._plan = staging.to_device(block, max(words.value, 1), indices.device)
         self._planned = True
 
+    def fused_append_supported(self, dtype: torch.dtype) -> bool:
+        """Whether forward(..., k_append=, v_append=) can write the step's token itself for
+        the shape given to begin_forward."""
+        if dtype not in (torch.bfloat16, torch.float16):
+            return False
+        return bool(_lib.lib().dskv_decode_append_attn_supported(self._hq, self._hkv, self._d, self._p,
+                                                                 _lib.dtype_code(dtype)))
+
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,
                 sm_scale: Optional[float] = None, *, phases: int = 3,
-                out: Optional[torch.Tensor] = None, **_ignored) -> torch.Tensor:
-        """phases: 1 = split-KV pass only, 2 = merge pass only, 3 = both (default)."""
+                out: Optional[torch.Tensor] = None, k_append: Optional[torch.Tensor] = None,
+                v_append: Optional[torch.Tensor] = None, **_ignored) -> torch.Tensor:
+        """phases: 1 = split-KV pass only, 2 = merge pass only, 3 = both (default).
+        k_append, v_append (batch, Hkv, D): the step's token of every request, not yet in the
+        pages - the attention launch writes them into their slots itself (one launch less than
+        append_paged_kv_cache + forward; see fused_append_supported)."""
         if not self._planned:
             raise RuntimeError("decode forward called before begin_forward")
         q = q.contiguous()
@@ -166,11 +178,28 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         if out is None:
             out = torch.empty_like(q)
         scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
+        ws_bytes = self._workspace.numel() * self._workspace.element_size()
+        if k_append is not None or v_append is not None:
+            if k_append is None or v_append is None or phases not in (1, 3):
+                raise ValueError("the fused form takes both k_append and v_append, with the attention pass")
+            k_append, v_append = k_append.contiguous(), v_append.contiguous()
+            want = (self._batch, self._hkv, self._d)
+            if tuple(k_append.shape) != want or tuple(v_append.shape) != want or \
+                    k_append.dtype != q.dtype or v_append.dtype != q.dtype:
+                raise ValueError(f"k_append / v_append must be {want} of q's dtype")
+            rc = _lib.lib().dskv_decode_append_attn(
+                out.data_ptr(), q.data_ptr(), k_append.data_ptr(), v_append.data_ptr(),
+                paged_kv_data.data_ptr(), self._indices.data_ptr(), self._plan.data_ptr(),
+                self._n_items, self._n_workgroups, self._workspace.data_ptr(), ws_bytes, self._batch,
+                self._hq, self._hkv, self._d, self._p, scale, _lib.dtype_code(q.dtype), phases,
+                _lib.current_stream())
+            _lib.check(rc, "decode append + forward")
+            return out
         rc = _lib.lib().dskv_decode_attn_phases(
             out.data_ptr(), q.data_ptr(), paged_kv_data.data_ptr(), self._indices.data_ptr(),
-            self._plan.data_ptr(), self._n_items, self._n_workgroups, self._workspace.data_ptr(), self._workspace.numel() * self._workspace.element_size(),
-            self._batch, self._hq, self._hkv, self._d, self._p, scale, _lib.dtype_code(q.dtype),
-            phases, _lib.current_stream())
+            self._plan.data_ptr(), self._n_items, self._n_workgroups, self._workspace.data_ptr(),
+            ws_bytes, self._batch, self._hq, self._hkv, self._d, self._p, scale,
+            _lib.dtype_code(q.dtype), phases, _lib.current_stream())
         _lib.check(rc, "decode forward")
         return out
 

@@ -123,6 +123,28 @@ int dskv_decode_attn_phases(void *out, const void *q, const void *pages_layer,
                             int32_t dtype, int32_t phases, void *stream);
 
 /*
+ * The decode step's append and attention in one launch (same plan, same result
+ * as dskv_append_paged_kv of one token per request followed by
+ * dskv_decode_attn; replaces the pair of calls of
+ * model/layer/attention.py:174-187 in a decode step).  k_new, v_new:
+ * (batch, n_kv_heads, head_dim), the step's token of every request; the plan's
+ * kv lengths include it and its page slot exists.  The wave that reads a
+ * request's newest row writes it first, so no other launch has to.  phases: 3,
+ * or 1 to leave the merge pass to a later dskv_decode_attn_phases(.., 2, ..).  Only for
+ * the shapes dskv_decode_append_attn_supported accepts (16-bit, head_dim 128,
+ * group <= 16, power-of-two page); others return DSKV_E_INVAL.
+ */
+int dskv_decode_append_attn_supported(int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                                      int32_t page_size, int32_t dtype);
+int dskv_decode_append_attn(void *out, const void *q, const void *k_new, const void *v_new,
+                            void *pages_layer, const int32_t *kv_page_indices,
+                            const int32_t *plan_dev, int32_t n_items, int32_t n_workgroups,
+                            void *workspace, int64_t workspace_bytes, int32_t batch,
+                            int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                            int32_t page_size, float sm_scale, int32_t dtype, int32_t phases,
+                            void *stream);
+
+/*
  * Paged prefill attention with the end-aligned causal mask.  Replaces
  * BatchPrefillWithPagedKVCacheWrapper.forward(q, pages, causal=True)
  * (model/layer/attention.py:188-192, execution/exec.py:227-236).

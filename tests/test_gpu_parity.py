@@ -318,6 +318,60 @@ def test_decode_attention_random_shapes():
         done += 1
 
 
+FUSED_CASES = [c for c in DECODE_CASES if c[6] in ("bf16", "f16") and c[5] == 128 and min(c[1]) >= 1]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES, ids=[c[0] for c in FUSED_CASES])
+def test_decode_with_fused_append_equals_append_then_decode(case):
+    """forward(k_append=, v_append=) leaves the pages as the oracle's append does and returns
+    bit for bit what append_paged_kv_cache + forward return."""
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper, append_paged_kv_cache
+
+    name, kv, P, Hq, Hkv, D, dtype, target = case
+    _announce("decode fused append", name)
+    sc = make_scenario(911, kv_lens=kv, qo_lens=[1] * len(kv), P=P, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype)
+    want_pages = sc.pages.copy()
+    orc.append_paged_kv(want_pages, sc.k, sc.v, sc.qo_indptr, sc.kv_page_indices, sc.kv_page_indptr,
+                        sc.kv_last_page_lens)
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
+    meta = (_dev_i32(sc.kv_page_indices), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_last_page_lens))
+    w.begin_forward(meta[1], meta[0], meta[2], Hq, Hkv, D, P, target_workgroups=target)
+    assert w.fused_append_supported(torch_dtype(dtype))
+    q, k, v = to_torch(sc.q, dtype), to_torch(sc.k, dtype), to_torch(sc.v, dtype)
+    pages_a, pages_b = to_torch(sc.pages, dtype), to_torch(sc.pages, dtype)
+    append_paged_kv_cache(k, v, _dev_i32(sc.qo_indptr), pages_a, *meta)
+    out_a = w.forward(q, pages_a)
+    out_b = w.forward(q, pages_b, k_append=k, v_append=v)
+    torch.cuda.synchronize()
+    assert _same_bits(from_torch(pages_b, dtype), want_pages) and _same_bits(from_torch(pages_a, dtype), want_pages)
+    assert _same_bits(from_torch(out_b, dtype), from_torch(out_a, dtype))
+    want = c_oracle.decode_attn(sc.q, want_pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                sc.kv_last_page_lens, dtype)
+    assert max_rel_err(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
+    with pytest.raises(ValueError):
+        w.forward(q, pages_b, k_append=k)
+    with pytest.raises(ValueError):
+        w.forward(q, pages_b, k_append=k[:, :1], v_append=v[:, :1])
+    w.end_forward()
+
+
+def test_fused_append_is_refused_outside_the_mfma_shapes():
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+
+    _announce("decode fused append refusal")
+    sc = make_scenario(912, kv_lens=[40, 3], qo_lens=[1, 1], P=16, Hq=8, Hkv=2, D=64, dtype="f32")
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    w.begin_forward(_dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                    _dev_i32(sc.kv_last_page_lens), 8, 2, 64, 16)
+    assert not w.fused_append_supported(torch.float32)
+    pages = to_torch(sc.pages, "f32")
+    before = from_torch(pages, "f32").copy()
+    with pytest.raises(ValueError, match="separately"):
+        w.forward(to_torch(sc.q, "f32"), pages, k_append=to_torch(sc.k, "f32"), v_append=to_torch(sc.v, "f32"))
+    torch.cuda.synchronize()
+    assert _same_bits(from_torch(pages, "f32"), before)
+
+
 def test_prefill_with_one_query_equals_decode():
     from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
 
