@@ -18,6 +18,7 @@ request x head) on a bounded sample, on this box's host cores.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -31,10 +32,19 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_BF16_TFLOPS = 2500.0
 
 
+def settle_heap():
+    """A full collection of the Python heap takes 20-40 ms in this process (170 k tracked
+    objects): one that happens to fall into a timed loop starves the GPU for that long.
+    Collect now and move what exists out of the collector's reach, as a long-running engine
+    does after start-up; what the steps allocate is still collected (cheaply)."""
+    gc.collect()
+    gc.freeze()
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
@@ -143,6 +153,7 @@ def swap_section(seed: int):
     nbytes = host_out.numel() * 2
     eng = _native.SwapEngine()
     w, _ = get_wrappers(wl.pool.main_device)
+    settle_heap()
 
     def decode_step():
         c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, w)
@@ -463,6 +474,7 @@ def main() -> int:
     wl = make_decode_workload("cfg2", ctx, L, Hq, Hkv, D, P, torch.bfloat16,
                               headroom_tokens=total_steps + 8, seed=a.seed, use_rope=a.rope)
     decode_wrapper, _ = get_wrappers(wl.pool.main_device)
+    settle_heap()
     e = wl.pool.pages.element_size()
     tok_bytes = wl.kv_bytes_per_token()
     torch.cuda.synchronize()
@@ -546,13 +558,16 @@ def main() -> int:
         return ev
 
     t0 = time.perf_counter()
+    marks = [t0]
     for i in range(a.steps):
         ev = wait_turn(i)
         last_ctx = one_step(True)
         if ev is not None:
             ev.record()
+        marks.append(time.perf_counter())
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    loop_ms = np.diff(np.array(marks)) * 1e3       # host time per loop turn (enqueue + its wait)
 
     ms_per_step = elapsed / a.steps * 1e3
     value = sum(step_bytes) / elapsed / 1e9
@@ -570,6 +585,8 @@ def main() -> int:
                    "append": "inside the attention launch" if fused else "own launch"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "stage_tokens_per_s": round(wl.batch / (elapsed / a.steps), 1),
+        "host_loop_ms": {"median": round(float(np.median(loop_ms)), 3), "max": round(float(loop_ms.max()), 3),
+                         "turns_over_3ms": int((loop_ms > 3.0).sum())},
     }
     if ev_pairs:
         all_ms = sorted(s.elapsed_time(t) for s, t in ev_pairs)
