@@ -128,6 +128,8 @@ DECODE_CASES = [
     ("f32_d64", [200, 17], 8, 8, 2, 64, "f32", 0),
     ("bf16_d64_generic", [200, 17], 16, 8, 2, 64, "bf16", 4),
     ("empty_request", [0, 50], 16, 32, 8, 128, "bf16", 0),
+    ("long_single", [33000], 16, 32, 8, 128, "bf16", 0),          # 256 parts: the wide merge
+    ("long_and_short", [9000, 50, 1], 16, 32, 8, 128, "f16", 128),
 ]
 
 
