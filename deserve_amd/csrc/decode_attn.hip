@@ -48,7 +48,10 @@ constexpr int kStages = DSKV_DECODE_STAGES;   // tiles in flight per wave (one c
 constexpr int kPlanHeaderWords = 4;  // n_items, n_workgroups, n_slots, batch
 constexpr int kItemWords = 8;
 constexpr int kMaxWorkgroups = 4096;
-constexpr int kMinTilesPerWorkgroup = 4;
+#ifndef DSKV_DECODE_MIN_TILES
+#define DSKV_DECODE_MIN_TILES 4
+#endif
+constexpr int kMinTilesPerWorkgroup = DSKV_DECODE_MIN_TILES;
 
 // Work item written by the planner.  slot < 0: the item covers its whole request
 // and writes the final output row; otherwise it writes partial slot `slot`.
