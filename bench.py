@@ -59,7 +59,7 @@ def parse_args():
                     help="steps the host may have queued on the GPU (a stage hands every step's "
                          "output on before it starts the next but one); 0 = no limit")
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
-    ap.add_argument("--section", choices=["swap", "fragmented"], default=None,
+    ap.add_argument("--section", choices=["swap", "fragmented", "prefill"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
@@ -448,7 +448,8 @@ def main() -> int:
     if a.section is not None:
         import torch
         torch.cuda.set_device(0)
-        print(json.dumps({"swap": swap_section, "fragmented": fragmented_section}[a.section](a.seed)))
+        print(json.dumps({"swap": swap_section, "fragmented": fragmented_section,
+                          "prefill": prefill_section}[a.section](a.seed)))
         return 0
     if a.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {a.gpus} is not supported in this build "
@@ -599,7 +600,38 @@ def main() -> int:
         tfile = os.path.join(ROOT, "profiles", "decode_attn_cfg2_traffic.json")
         if os.path.exists(tfile):
             traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
+        # cross-checks of the bracketed figure: what a bracket costs with nothing inside it, and
+        # the same pass over all layers back to back inside ONE bracket (no cache reuse between
+        # layers); bracket - empty bracket, the back-to-back time and rocprofv3 agree
+        empty = []
+        for _ in range(21):
+            s, t = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            wl.q[0].mul_(1.0)                                # the brackets follow work, as in a step
+            s.record()
+            t.record()
+            empty.append((s, t))
+        c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, decode_wrapper)
+        decode_wrapper.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
+                                     last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
+                                     num_kv_heads=Hkv, head_dim=D, page_size=P,
+                                     indptr_host=c.host["kv_page_indptr"],
+                                     last_page_len_host=c.host["kv_last_page_lens"],
+                                     target_workgroups=a.workgroups)
+        scratch_out = torch.empty_like(wl.q[0])
+        rounds = 3
+        s, t = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for r in range(rounds + 1):
+            if r == 1:
+                s.record()
+            for layer in range(L):
+                decode_wrapper.forward(wl.q[layer], wl.pool.get_layered_pages(layer), phases=1, out=scratch_out)
+        t.record()
+        decode_wrapper.end_forward()
+        torch.cuda.synchronize()
+        empty_us = sorted(x.elapsed_time(y) for x, y in empty)[len(empty) // 2] * 1e3
+        b2b_us = s.elapsed_time(t) * 1e3 / (rounds * L)
         out["roofline"] = {"bound": "hbm", "kernel": "decode_attn_mfma_kernel<bf16> (split-KV pass" + (", writes the step's token first)" if fused else ")"),
+                           "empty_bracket_us": round(empty_us, 2), "back_to_back_us": round(b2b_us, 2),
                            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                            "avg_launch_us": round(avg_ms * 1e3, 2), "launches": len(times_ms),
