@@ -135,7 +135,6 @@ def swap_section(seed: int):
     from deserve_amd.kvcache import _native
     from deserve_amd.kvcache.pinned.pinned_memory import pinned_empty
     from deserve_amd.model.context.flash import FlashDecodeCtx
-    from deserve_amd.paged_ops import append_paged_kv_cache
     from deserve_amd.synthetic import make_decode_workload
 
     L, Hq, Hkv, D, P = 10, 64, 8, 128, 16
@@ -163,9 +162,7 @@ def swap_section(seed: int):
                         last_page_len_host=c.host["kv_last_page_lens"])
         for layer in range(L):
             pages = wl.pool.get_layered_pages(layer)
-            append_paged_kv_cache(wl.k[layer], wl.v[layer], c.indptr, pages, c.kv_page_indices,
-                                  c.kv_page_indptr, c.kv_last_page_lens)
-            w.forward(wl.q[layer], pages)
+            w.forward(wl.q[layer], pages, k_append=wl.k[layer], v_append=wl.v[layer])
         w.end_forward()
         for t in wl.tasks:
             t.step()
@@ -325,7 +322,6 @@ def fragmented_section(seed: int):
     from deserve_amd.kvcache.paged.page_table import PageTableAllocator
     from deserve_amd.kvcache.virtual import VirtualPagedKVCache, VirtualPagePool
     from deserve_amd.model.context.flash import FlashDecodeCtx
-    from deserve_amd.paged_ops import append_paged_kv_cache
     from deserve_amd.synthetic import config5_context_lengths, fill_normal
     from deserve_amd.task import SamplingParams, TaskData
 
@@ -389,17 +385,16 @@ def fragmented_section(seed: int):
                         last_page_len_host=c.host["kv_last_page_lens"])
         for layer in range(L):
             pages = pool.get_layered_pages(layer)
-            append_paged_kv_cache(k[layer], v[layer], c.indptr, pages, c.kv_page_indices,
-                                  c.kv_page_indptr, c.kv_last_page_lens)
+            new_kv = dict(k_append=k[layer], v_append=v[layer])   # written by the attention launch
             if record and layer % 2 == 0:
                 s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 s.record()
-                out = w.forward(q[layer], pages, phases=1)
+                out = w.forward(q[layer], pages, phases=1, **new_kv)
                 e.record()
                 w.forward(q[layer], pages, phases=2, out=out)
                 ev.append((s, e))
             else:
-                w.forward(q[layer], pages)
+                w.forward(q[layer], pages, **new_kv)
         w.end_forward()
         if record:
             kv_lens = np.array([t.start_pos + 1 for t in tasks], dtype=np.int64)

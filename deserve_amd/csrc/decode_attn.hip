@@ -692,8 +692,10 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
     }
     if ((phases & 2) && n_items > batch) {
         dim3 grid((unsigned)batch, (unsigned)n_qo_heads);
-        // many parts per request (long requests, small batch): eight waves share a merge
-        const bool wide = (int64_t)n_items > 8 * (int64_t)batch;
+        // many parts per request (long requests, small batch): eight waves share a merge.
+        // One wave needs a round trip per 8 parts, eight waves a barrier and a second pass
+        // through LDS: they break even at about 32 parts.
+        const bool wide = (int64_t)n_items > 32 * (int64_t)batch;
 #define DSKV_LAUNCH_MERGE(DT)                                                                     \
     do {                                                                                          \
         if (wide)                                                                                 \
