@@ -177,26 +177,37 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             pg[i] = __builtin_amdgcn_raw_buffer_load_b32(page_table, (tok0 >> page_shift) * 4 + lane * 0, 0, 0);
         }
     };
-    auto load_rows = [&](int blk, const int(&pg)[kRowGroups], u32x4(&k_rows)[kRowGroups],
-                         u32x4(&v_rows)[kRowGroups]) {
+    // The descriptors of the rows of block blk (scalar work: page id into an SGPR, base
+    // address, valid bytes), prepared an iteration before the loads are issued so that it
+    // runs in the shadow of that iteration's MFMAs.
+    struct RowDesc {
+        __amdgpu_buffer_rsrc_t k[kRowGroups], v[kRowGroups];
+    };
+    auto prepare_rows = [&](int blk, const int(&pg)[kRowGroups], RowDesc &d) {
+        if (!kRowsSharePage) return;
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
             const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
+            // one page holds the 4 rows: descriptors that end after the last
+            // valid row make the bounds check free and keep offsets constant
+            const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
+            const long page = __builtin_amdgcn_readfirstlane(pg[i]);
+            char *first_row = const_cast<char *>(pages) + page * page_bytes +
+                              (long)(tok0 & page_mask) * row_bytes;
+            d.k[i] = __builtin_amdgcn_make_buffer_rsrc(first_row, 0, valid * row_bytes, kBufferFlags);
+            d.v[i] = __builtin_amdgcn_make_buffer_rsrc(first_row + half_bytes, 0, valid * row_bytes,
+                                                       kBufferFlags);
+        }
+    };
+    auto load_rows = [&](int blk, const RowDesc &d, u32x4(&k_rows)[kRowGroups],
+                         u32x4(&v_rows)[kRowGroups]) {
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++) {
             if (kRowsSharePage) {
-                // one page holds the 4 rows: descriptors that end after the last
-                // valid row make the bounds check free and keep offsets constant
-                const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
-                const long page = __builtin_amdgcn_readfirstlane(pg[i]);
-                char *first_row = const_cast<char *>(pages) + page * page_bytes +
-                                  (long)(tok0 & page_mask) * row_bytes;
-                __amdgpu_buffer_rsrc_t k_desc = __builtin_amdgcn_make_buffer_rsrc(
-                    first_row, 0, valid * row_bytes, kBufferFlags);
-                __amdgpu_buffer_rsrc_t v_desc = __builtin_amdgcn_make_buffer_rsrc(
-                    first_row + half_bytes, 0, valid * row_bytes, kBufferFlags);
-                k_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(k_desc, lane_off, 0, kLoadCached);
-                v_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(v_desc, lane_off, 0, kLoadCached);
+                k_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(d.k[i], lane_off, 0, kLoadCached);
+                v_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(d.v[i], lane_off, 0, kLoadCached);
             } else {
-                const int tok = tok0 + g;
+                const int tok = blk * kBlock + wave * kRowsPerWave + 4 * i + g;
                 const int tc = min(tok, t_end - 1);
                 const char *p = pages + page_ids[tc >> page_shift] * page_bytes +
                                 (long)(tc & page_mask) * row_bytes + (lane_off - g * row_bytes);
@@ -276,8 +287,9 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     // P(m) and computes S(m+1), so that every MFMA of the iteration is independent
     // of its exponentials and the matrix and vector pipelines of a wave overlap.
     // The rows of block m+4 are requested in iteration m (their page id was looked
-    // up in iteration m-2) and written to LDS in iteration m+2: one iteration is
-    // shorter than a trip to memory.  K has two LDS stages and V four (V(j) is
+    // up in iteration m-2, their descriptors built in iteration m-1 behind its
+    // MFMAs) and written to LDS in iteration m+2: one iteration is shorter than a
+    // trip to memory.  K has two LDS stages and V four (V(j) is
     // read three iterations after it is stored).  Per iteration one barrier: past
     // it K(m+1) and V(m-1) are complete and the stages of K(m) and V(m-2) are free.
     // Every wave runs every iteration (idle ones only move rows), so the barriers
@@ -285,6 +297,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     struct RowSet {
         u32x4 k[kRowGroups], v[kRowGroups];   // rows on their way to LDS
         int pg[kRowGroups];                   // page ids of the rows requested next
+        RowDesc desc;                         // their descriptors, once prepared
     };
     RowSet even, odd;
     {
@@ -292,8 +305,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
 #pragma unroll
         for (int blk = 0; blk < 2; blk++) {
+            RowDesc d;
             lookup_pages(blk, pg);
-            load_rows(blk, pg, first_k[blk], first_v[blk]);
+            prepare_rows(blk, pg, d);
+            load_rows(blk, d, first_k[blk], first_v[blk]);
         }
         lookup_pages(2, even.pg);
         lookup_pages(3, odd.pg);
@@ -308,10 +323,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             store_rows(v_stage[blk], kPVPitch, first_v[blk]);
         }
     }
-    load_rows(2, even.pg, even.k, even.v);
-    load_rows(3, odd.pg, odd.k, odd.v);
+    prepare_rows(2, even.pg, even.desc);
+    prepare_rows(3, odd.pg, odd.desc);
+    load_rows(2, even.desc, even.k, even.v);
+    load_rows(3, odd.desc, odd.k, odd.v);
     lookup_pages(4, even.pg);
     lookup_pages(5, odd.pg);
+    prepare_rows(4, even.pg, even.desc);   // iteration 0 issues these; every iteration prepares the next one's
     __syncthreads();
     if (w_end > 0) {
         read_k_operands(k_stage[0]);
@@ -320,13 +338,16 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         block_max();
     }
     const int v_lane_off = (4 * h + (c >> 2)) * kPVPitch + (g & 1) * 32 + (c & 3) * 8;
-    auto iteration = [&](int m, int phase, RowSet &rows) {   // phase = m % 4, a literal at each call
+    auto iteration = [&](int m, int phase, RowSet &rows, RowSet &next) {   // phase = m % 4, a literal at each call
         __syncthreads();
         store_rows(k_stage[phase & 1], kKPitch, rows.k);              // K(m+2)
         store_rows(v_stage[(phase + 2) & 3], kPVPitch, rows.v);       // V(m+2)
-        load_rows(m + 4, rows.pg, rows.k, rows.v);
+        load_rows(m + 4, rows.desc, rows.k, rows.v);
         lookup_pages(m + 6, rows.pg);
-        if (!(w_end > 0 && (m - 1) * kBlock < w_end)) return;
+        if (!(w_end > 0 && (m - 1) * kBlock < w_end)) {
+            prepare_rows(m + 5, next.pg, next.desc);
+            return;
+        }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
             // rare: raise the maximum and bring what was computed under the old
             // one (accumulators, row sum, the pending P(m-1)) to the new scale
@@ -406,15 +427,16 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ct++)
                     acc[ct][dt] = E::mfma_32x32(va[dt][ks], pb_prev[ct][ks], acc[ct][dt]);
+        prepare_rows(m + 5, next.pg, next.desc);   // for the loads of the next iteration
         block_max();
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
     };
     for (int m = 0; m <= n_blocks; m += 4) {
-        iteration(m, 0, even);
-        iteration(m + 1, 1, odd);
-        iteration(m + 2, 2, even);
-        iteration(m + 3, 3, odd);
+        iteration(m, 0, even, odd);
+        iteration(m + 1, 1, odd, even);
+        iteration(m + 2, 2, even, odd);
+        iteration(m + 3, 3, odd, even);
     }
 
 #pragma unroll
