@@ -49,6 +49,18 @@ def test_argument_errors_return_negative_codes_without_a_gpu():
     assert "power-of-two" in _lib.last_error()
     assert lib.dskv_decode_attn(16, 16, 16, 16, 16, 2, 0, None, 0, 2, 32, 8, 128, 16, 0.1, 2, None) == -1
     assert lib.dskv_decode_attn_phases(16, 16, 16, 16, 16, 2, 2, None, 0, 2, 32, 8, 128, 16, 0.1, 2, 0, None) == -1
+    # out, q, k_new, v_new, pages, indices, plan, n_items, n_wgs, ws, ws_bytes, batch, Hq, Hkv, D, P, scale, dtype, phases, stream
+    fused = (16, 16, 16, 16, 16, 16, 16, 2, 2, None, 0, 2, 32, 8, 128, 16, 0.1)
+    assert lib.dskv_decode_append_attn(*fused, 2, 2, None) == -1 and "phases" in _lib.last_error()
+    assert lib.dskv_decode_append_attn(16, 16, None, 16, *fused[4:], 2, 3, None) == -1
+    assert lib.dskv_decode_append_attn(16, 16, 16, 24, *fused[4:], 2, 3, None) == -1 and "aligned" in _lib.last_error()
+    assert lib.dskv_decode_append_attn(*fused, 0, 3, None) == -1 and "separately" in _lib.last_error()   # fp32
+    assert lib.dskv_decode_append_attn(*fused[:11], 0, *fused[12:], 2, 3, None) == 0                    # empty batch
+    assert lib.dskv_decode_append_attn_supported(32, 8, 128, 16, 2) == 1
+    assert lib.dskv_decode_append_attn_supported(32, 8, 128, 16, 0) == 0      # fp32 pool
+    assert lib.dskv_decode_append_attn_supported(32, 8, 64, 16, 2) == 0       # head_dim
+    assert lib.dskv_decode_append_attn_supported(32, 8, 128, 12, 2) == 0      # page size
+    assert lib.dskv_decode_append_attn_supported(64, 2, 128, 16, 1) == 0      # group of 32
     assert lib.dskv_apply_rope(16, 16, 16, 16, 16, 16, 1, 1, 32, 8, 130, 5e5, 2, None) == -1
     assert lib.dskv_upload_words(16, 16, -1, None) == -1 and lib.dskv_upload_words(None, None, 0, None) == 0
     assert lib.dskv_upload_words(16, 24, 4, None) == -1 and "16-byte" in _lib.last_error()
