@@ -6,7 +6,8 @@ captures what ``layer_storage.forward(xs, ctx)`` launches for one batch shape
 into a graph and replays it: per step the host only rebuilds the CSR metadata
 and the split-KV work list in pinned buffers that never move, copies both to
 device buffers that never move, and replays.  A new batch size (or workgroup
-count) triggers a new capture.
+count) triggers a new capture; the last few captures are kept, so a scheduler that
+alternates between batch sizes replays instead of capturing again.
 
 Nothing that is captured clears memory with a memset node, and the library
 calls allocate nothing; the outputs of the captured forward live in the graph's
@@ -14,6 +15,7 @@ own memory pool and are overwritten by every replay.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from typing import List, Sequence
 
 import torch
@@ -28,7 +30,7 @@ from deserve_amd.task import TaskData
 class GraphedDecodeStep:
     def __init__(self, layer_storage, wrapper: BatchDecodeWithPagedKVCacheWrapper, max_batch: int,
                  max_pages: int, device: torch.device, num_qo_heads: int, num_kv_heads: int,
-                 head_dim: int, page_size: int, target_workgroups: int = 0) -> None:
+                 head_dim: int, page_size: int, target_workgroups: int = 0, max_graphs: int = 8) -> None:
         self.layer_storage, self.wrapper = layer_storage, wrapper
         self.shape = dict(num_qo_heads=num_qo_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
                           page_size=page_size)
@@ -36,8 +38,9 @@ class GraphedDecodeStep:
         self.meta = MetadataBuffers(max_batch, max_pages, device)
         words = int(_lib.lib().dskv_decode_plan_bound(max_batch, max_pages * page_size))
         self.plan = StagedUpload(words, device)
-        self._key = None
-        self._graph = None
+        self.max_graphs = max_graphs
+        self._graphs: "OrderedDict[tuple, tuple]" = OrderedDict()   # key -> (graph, inputs, output)
+        self._graph = None                     # the one replayed last
         self._inputs: List[torch.Tensor] = []
         self._output = None
         self.captures = 0
@@ -58,21 +61,30 @@ class GraphedDecodeStep:
         tensors = list(xs) if isinstance(xs, (tuple, list)) else [xs]
         ctx = self._prepare(task_datas, kvcaches)
         w = self.wrapper
-        key = (len(task_datas), w._n_workgroups, w._n_items > len(task_datas),
+        # what decides which kernels a step launches: batch, workgroups, whether anything is
+        # merged and with which of the two merge kernels (the launcher takes the wide one
+        # from 32 parts per request on)
+        batch = len(task_datas)
+        key = (batch, w._n_workgroups, w._n_items > batch, w._n_items > 32 * batch,
                tuple((tuple(t.shape), t.dtype) for t in tensors))
-        if key != self._key:
-            self._inputs = [t.clone() for t in tensors]
-            static = tuple(self._inputs) if isinstance(xs, (tuple, list)) else self._inputs[0]
+        held = self._graphs.get(key)
+        if held is None:
+            inputs = [t.clone() for t in tensors]
+            static = tuple(inputs) if isinstance(xs, (tuple, list)) else inputs[0]
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                self._output = self.layer_storage.forward(static, ctx)
-            self._graph, self._key = graph, key
+                output = self.layer_storage.forward(static, ctx)
+            self._graphs[key] = held = (graph, inputs, output)
             self.captures += 1
+            while len(self._graphs) > self.max_graphs:
+                self._graphs.popitem(last=False)        # least recently used
         else:
+            self._graphs.move_to_end(key)
             # one copy kernel on the launch stream for all inputs: device-to-device memcpy
             # calls may go through a DMA engine, whose hand-over to and from the compute
             # queue costs more than the copies themselves
-            torch._foreach_copy_(self._inputs, tensors)
+            torch._foreach_copy_(held[1], tensors)
+        self._graph, self._inputs, self._output = held
         self._graph.replay()
         w.end_forward()
         return self._output

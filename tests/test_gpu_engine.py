@@ -299,7 +299,7 @@ def test_graphed_decode_step_matches_eager_steps():
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16))
-    assert step.captures == 2
+    assert step.captures == 2 and len(step._graphs) == 2       # both batch shapes are held for replay
 
 
 @pytest.mark.gpu
