@@ -48,7 +48,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seed", type=int, default=2)
     ap.add_argument("--workgroups", type=int, default=0, help="persistent workgroups of the attention pass (0 = one per CU)")
-    ap.add_argument("--rope", action="store_true", help="also apply RoPE to q/k before the append")
+    ap.add_argument("--rope", action="store_true", help="also rotate q and k (RoPE) in the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-swap", action="store_true", help="skip the microbatch swap section")
     ap.add_argument("--no-prefill", action="store_true", help="skip the chunked-prefill section")
@@ -457,7 +457,7 @@ def main() -> int:
     from deserve_amd import _lib
     from deserve_amd.execution.exec import get_wrappers
     from deserve_amd.model.context.flash import FlashDecodeCtx
-    from deserve_amd.paged_ops import append_paged_kv_cache, apply_rope
+    from deserve_amd.paged_ops import append_paged_kv_cache, rope_append_paged_kv_cache
     from deserve_amd.synthetic import config2_context_lengths, make_decode_workload
 
     if not os.path.exists(_lib.LIB_PATH):
@@ -494,7 +494,7 @@ def main() -> int:
     step_bytes = []
     attn_bytes_layer = []
 
-    fused = not a.no_fused_append and not a.rope
+    fused = not a.no_fused_append
 
     def one_step(timed: bool):
         """prepare (metadata + plan, one upload each) then L x (append + attention: one launch
@@ -508,15 +508,20 @@ def main() -> int:
                                      target_workgroups=a.workgroups)
         for layer in range(L):
             q, k, v = wl.q[layer], wl.k[layer], wl.v[layer]
-            if a.rope:
-                q, k = apply_rope(q, k, c.indptr, c.offsets, interleave=True, rope_theta=5e5)
             pages = wl.pool.get_layered_pages(layer)
             if fused:
-                new_kv = dict(k_append=k, v_append=v)    # the attention launch writes the token
+                # the attention launch (rotates q and k and) writes the token
+                new_kv = dict(k_append=k, v_append=v)
+                if a.rope:
+                    new_kv.update(rope_offsets=c.offsets, rope_theta=5e5)
             else:
                 new_kv = {}
-                append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
-                                      c.kv_last_page_lens)
+                if a.rope:
+                    q = rope_append_paged_kv_cache(q, k, v, c.indptr, c.offsets, pages, c.kv_page_indices,
+                                                   c.kv_page_indptr, c.kv_last_page_lens, rope_theta=5e5)
+                else:
+                    append_paged_kv_cache(k, v, c.indptr, pages, c.kv_page_indices, c.kv_page_indptr,
+                                          c.kv_last_page_lens)
             launch_no[0] += 1
             if timed and not a.no_kernel_events and launch_no[0] % max(a.event_every, 1) == 0:
                 s, t = ev_pool[len(ev_pairs)]

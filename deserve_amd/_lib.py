@@ -46,6 +46,11 @@ _SIGNATURES = {
                                           c_void_p, c_int32, c_int32, c_void_p, c_int64, c_int32,
                                           c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
                                           c_int32, c_void_p]),
+    "dskv_rope_table": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_float, c_void_p]),
+    "dskv_decode_rope_append_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                               c_void_p, c_void_p, c_int32, c_int32, c_void_p,
+                                               c_int64, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                               c_float, c_int32, c_void_p, c_int32, c_void_p]),
     "dskv_prefill_plan_bound": (c_int64, [c_int32, c_int64]),
     "dskv_prefill_plan": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_int64,
                                     POINTER(c_int32)]),

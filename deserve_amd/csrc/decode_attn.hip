@@ -33,6 +33,7 @@
 //     needs 4 tokens of ONE dim per lane - the transpose of how it lies in
 //     memory - so the V tile goes through a wave-private LDS tile.
 #include "kv_tile.h"
+#include "rope_math.h"
 
 #include <algorithm>
 #include <math.h>
@@ -86,7 +87,8 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     const int32_t *__restrict__ kv_indices, const Item *__restrict__ items,
     const int32_t *__restrict__ wg_ptr, float *__restrict__ part_o, float *__restrict__ part_ml,
     int max_slots, int n_qo_heads, int n_kv_heads, int page_shift, float scale_log2,
-    const uint16_t *__restrict__ k_new, const uint16_t *__restrict__ v_new)
+    const uint16_t *__restrict__ k_new, const uint16_t *__restrict__ v_new,
+    const float *__restrict__ rope)
 {
     typedef Elt<DT> E;
     __shared__ __align__(16) char v_lds[kMaxWaves][kVTileBytes];
@@ -132,24 +134,62 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
             char *row = const_cast<char *>(pages) + page * kv.page_bytes +
                         (long)(tok & ((1 << page_shift) - 1)) * kv.row_bytes + kv.head_off;
             const long src = ((long)it.b * n_kv_heads + kvh) * kHeadDim;
-            if (lane < 16)
-                *reinterpret_cast<u32x4 *>(row + lane * 16) =
-                    *reinterpret_cast<const u32x4 *>(k_new + src + lane * 8);
-            else if (lane < 32)
+            if (lane < 16) {
+                u32x4 chunk = *reinterpret_cast<const u32x4 *>(k_new + src + lane * 8);
+                if (rope) {   // dims 8*lane .. +7 = pairs 4*lane .. +3 of the request's position
+                    const float *tab = rope + (long)it.b * kHeadDim + lane * 4;
+                    const f32x4 cs = *reinterpret_cast<const f32x4 *>(tab);
+                    const f32x4 sn = *reinterpret_cast<const f32x4 *>(tab + kHeadDim / 2);
+                    const float c4[4] = {cs[0], cs[1], cs[2], cs[3]}, s4[4] = {sn[0], sn[1], sn[2], sn[3]};
+                    float f[8];
+                    Chunk<DT>::unpack(chunk, f);
+                    rope_rotate<4>(f, c4, s4);
+                    chunk = Chunk<DT>::pack(f);
+                }
+                *reinterpret_cast<u32x4 *>(row + lane * 16) = chunk;
+            } else if (lane < 32)
                 *reinterpret_cast<u32x4 *>(row + kv.half_bytes + (lane - 16) * 16) =
                     *reinterpret_cast<const u32x4 *>(v_new + src + (lane - 16) * 8);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 
-    // Q rows of one item as the B operand of the score MFMAs (zero beyond the group).
-    auto load_q = [&](int item_idx, u32x4 (&dst)[4]) {
+    // Q rows of one item as the B operand of the score MFMAs (zero beyond the group), and,
+    // with a rope table, the cosines and sines of the lane's 16 dim pairs at the request's
+    // position.  finish_q turns the two into the operand once they have arrived.
+    struct QRaw {
+        u32x4 q[4];
+        f32x4 cs[4], sn[4];
+    };
+    auto load_q = [&](int item_idx, QRaw &dst) {
         const int b = item_words[(long)item_idx * kItemWords];
         const uint16_t *qrow = q + ((long)b * n_qo_heads + (long)kvh * group + c) * kHeadDim + g * 8;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             u32x4 z = {0, 0, 0, 0};
-            dst[kk] = (c < group) ? *reinterpret_cast<const u32x4 *>(qrow + kk * 32) : z;
+            dst.q[kk] = (c < group) ? *reinterpret_cast<const u32x4 *>(qrow + kk * 32) : z;
+        }
+        if (rope) {
+            const float *tab = rope + (long)b * kHeadDim + g * 4;   // dims 32*kk + 8*g .. +7
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                dst.cs[kk] = *reinterpret_cast<const f32x4 *>(tab + kk * 16);
+                dst.sn[kk] = *reinterpret_cast<const f32x4 *>(tab + kHeadDim / 2 + kk * 16);
+            }
+        }
+    };
+    auto finish_q = [&](const QRaw &raw, u32x4 (&dst)[4]) {
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            dst[kk] = raw.q[kk];
+            if (rope) {
+                const float c4[4] = {raw.cs[kk][0], raw.cs[kk][1], raw.cs[kk][2], raw.cs[kk][3]};
+                const float s4[4] = {raw.sn[kk][0], raw.sn[kk][1], raw.sn[kk][2], raw.sn[kk][3]};
+                float f[8];
+                Chunk<DT>::unpack(raw.q[kk], f);
+                rope_rotate<4>(f, c4, s4);
+                dst[kk] = Chunk<DT>::pack(f);
+            }
         }
     };
 
@@ -183,8 +223,9 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
         settle();
     };
 
-    u32x4 qreg[4], qnext[4];
-    load_q(item_begin, qreg);
+    u32x4 qreg[4];
+    QRaw qnext;
+    load_q(item_begin, qnext);
     settle();
     TileRegs ring[kStages];
 #pragma unroll
@@ -196,6 +237,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
         const int t_end = item.tok_end;
         // Q of the following item: issued now, so that it is older than every
         // tile load still in flight when it is needed (no drain at the switch)
+        if (idx == item_begin) finish_q(qnext, qreg);
         load_q(min(idx + 1, item_end - 1), qnext);
 
         f32x4 acc[8];
@@ -279,8 +321,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
                 }
             }
         }
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) qreg[kk] = qnext[kk];
+        finish_q(qnext, qreg);
     }
 }
 
@@ -608,7 +649,7 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
                             int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
                             int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
                             float sm_scale, int32_t dtype, int32_t phases, void *stream,
-                            const void *k_new, const void *v_new)
+                            const void *k_new, const void *v_new, const float *rope_table)
 {
     DSKV_REQUIRE(phases >= 1 && phases <= 3, "decode_attn: phases must be 1, 2 or 3");
     DSKV_REQUIRE(batch >= 0 && n_items >= 0 && n_workgroups >= 0,
@@ -668,7 +709,7 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
     hipLaunchKernelGGL((decode_attn_mfma_kernel<DT, COVER>), grid, block, 0, s, (uint16_t *)out, \
                        (const uint16_t *)q, (const char *)pages_layer, kv_page_indices, items,   \
                        wg_ptr, part_o, part_ml, (int)max_slots, n_qo_heads, n_kv_heads, shift,   \
-                       scale_log2, (const uint16_t *)k_new, (const uint16_t *)v_new)
+                       scale_log2, (const uint16_t *)k_new, (const uint16_t *)v_new, rope_table)
         if (dtype == DSKV_BF16) {
             if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_BF16, true);
             else DSKV_LAUNCH_MFMA(DSKV_BF16, false);
@@ -726,7 +767,7 @@ extern "C" int dskv_decode_attn_phases(void *out, const void *q, const void *pag
     return dskv::decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items,
                                   n_workgroups, workspace, workspace_bytes, batch, n_qo_heads,
                                   n_kv_heads, head_dim, page_size, sm_scale, dtype, phases, stream,
-                                  nullptr, nullptr);
+                                  nullptr, nullptr, nullptr);
 }
 
 extern "C" int dskv_decode_append_attn_supported(int32_t n_qo_heads, int32_t n_kv_heads,
@@ -754,7 +795,29 @@ extern "C" int dskv_decode_append_attn(void *out, const void *q, const void *k_n
                  "decode_append_attn: k_new / v_new must be 16-byte aligned");
     return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
                             workspace, workspace_bytes, batch, n_qo_heads, n_kv_heads, head_dim,
-                            page_size, sm_scale, dtype, phases, stream, k_new, v_new);
+                            page_size, sm_scale, dtype, phases, stream, k_new, v_new, nullptr);
+}
+
+extern "C" int dskv_decode_rope_append_attn(void *out, const void *q, const void *k_new,
+                                            const void *v_new, void *pages_layer,
+                                            const int32_t *kv_page_indices, const int32_t *plan_dev,
+                                            int32_t n_items, int32_t n_workgroups, void *workspace,
+                                            int64_t workspace_bytes, int32_t batch,
+                                            int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                                            int32_t page_size, float sm_scale, int32_t dtype,
+                                            const float *rope_table, int32_t phases, void *stream)
+{
+    using namespace dskv;
+    if (batch == 0 || n_items == 0) return 0;
+    DSKV_REQUIRE(phases == 1 || phases == 3,
+                 "decode_rope_append_attn: rotation and append belong to the attention pass "
+                 "(phases 1 or 3)");
+    DSKV_REQUIRE(k_new && v_new && rope_table, "decode_rope_append_attn: null k_new / v_new / table");
+    DSKV_REQUIRE(((uintptr_t)k_new | (uintptr_t)v_new | (uintptr_t)rope_table) % 16 == 0,
+                 "decode_rope_append_attn: k_new / v_new / table must be 16-byte aligned");
+    return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
+                            workspace, workspace_bytes, batch, n_qo_heads, n_kv_heads, head_dim,
+                            page_size, sm_scale, dtype, phases, stream, k_new, v_new, rope_table);
 }
 
 extern "C" int dskv_decode_attn(void *out, const void *q, const void *pages_layer,

@@ -4,61 +4,9 @@
 // Elementwise, HBM-bound; one workgroup per token.  A thread owns one 16-byte
 // chunk column of the head dimension, evaluates its sin/cos once and walks the
 // heads, so the transcendental work is per (token, dim pair), not per head.
-#include "common.h"
-
-#include <math.h>
+#include "rope_math.h"
 
 namespace dskv {
-
-template <int DT> struct Chunk;   // 16 bytes <-> fp32 lanes
-template <> struct Chunk<DSKV_F32> {
-    static constexpr int kElems = 4;
-    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
-        const f32x4 v = __builtin_bit_cast(f32x4, raw);
-        f[0] = v.x;
-        f[1] = v.y;
-        f[2] = v.z;
-        f[3] = v.w;
-    }
-    static __device__ __forceinline__ u32x4 pack(const float *f) {
-        const f32x4 v = {f[0], f[1], f[2], f[3]};
-        return __builtin_bit_cast(u32x4, v);
-    }
-};
-template <> struct Chunk<DSKV_F16> {
-    static constexpr int kElems = 8;
-    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-    typedef float f8 __attribute__((ext_vector_type(8)));
-    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
-        const f8 v = __builtin_convertvector(__builtin_bit_cast(h8, raw), f8);
-        f[0] = v.s0; f[1] = v.s1; f[2] = v.s2; f[3] = v.s3;
-        f[4] = v.s4; f[5] = v.s5; f[6] = v.s6; f[7] = v.s7;
-    }
-    static __device__ __forceinline__ u32x4 pack(const float *f) {
-        const f8 v = {f[0], f[1], f[2], f[3], f[4], f[5], f[6], f[7]};
-        return __builtin_bit_cast(u32x4, __builtin_convertvector(v, h8));
-    }
-};
-template <> struct Chunk<DSKV_BF16> {
-    static constexpr int kElems = 8;
-    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-    static __device__ __forceinline__ void unpack(u32x4 raw, float *f) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            f[2 * i] = __builtin_bit_cast(float, raw[i] << 16);
-            f[2 * i + 1] = __builtin_bit_cast(float, raw[i] & 0xFFFF0000u);
-        }
-    }
-    static __device__ __forceinline__ u32x4 pack(const float *f) {
-        u32x4 r;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            b2 p = {(__bf16)f[2 * i], (__bf16)f[2 * i + 1]};
-            r[i] = __builtin_bit_cast(uint32_t, p);
-        }
-        return r;
-    }
-};
 
 // Where the fused variant puts the rotated K row and the V row of a token: the
 // page slot the append would have chosen (see append.hip).
@@ -111,12 +59,7 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
 
     float cs[E / 2], sn[E / 2];
 #pragma unroll
-    for (int j = 0; j < E / 2; j++) {
-        const int pair = col * (E / 2) + j;
-        // theta^(-2*pair/D), evaluated as the reference's table does: 1 / theta^(2*pair/D)
-        const float inv_freq = 1.0f / powf(theta, (float)(2 * pair) / (float)head_dim);
-        sincosf(pos * inv_freq, &sn[j], &cs[j]);
-    }
+    for (int j = 0; j < E / 2; j++) rope_angle(pos, col * (E / 2) + j, head_dim, theta, cs[j], sn[j]);
     const long row_bytes = (long)head_dim * (16 / E);
     const int total_heads = n_qo_heads + n_kv_heads;
     for (int h = head_lane; h < total_heads; h += head_lanes) {
@@ -128,12 +71,7 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
                          : k_dst + (long)(h - n_qo_heads) * row_bytes + col * 16;
         float f[E];
         C::unpack(*reinterpret_cast<const u32x4 *>(src), f);
-#pragma unroll
-        for (int j = 0; j < E / 2; j++) {
-            const float re = f[2 * j], im = f[2 * j + 1];
-            f[2 * j] = re * cs[j] - im * sn[j];
-            f[2 * j + 1] = re * sn[j] + im * cs[j];
-        }
+        rope_rotate<E / 2>(f, cs, sn);
         *reinterpret_cast<u32x4 *>(dst) = C::pack(f);
     }
     if (v_dst) {   // fused append: V rows are copied as they are
@@ -141,6 +79,22 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
         for (long off = threadIdx.x * 16L; off < kv_row_bytes; off += 256 * 16)
             *reinterpret_cast<u32x4 *>(v_dst + off) = *reinterpret_cast<const u32x4 *>(v_src + off);
     }
+}
+
+// cos | sin of every (request, dim pair) of a decode step: table[b][0 .. D/2) = cos,
+// table[b][D/2 .. D) = sin of positions[b] * theta^(-2*pair/D).
+__global__ __launch_bounds__(256) void rope_table_kernel(float *__restrict__ table,
+                                                         const int32_t *__restrict__ positions,
+                                                         int batch, int head_dim, float theta)
+{
+    const int pairs = head_dim / 2;
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)batch * pairs) return;
+    const int b = (int)(i / pairs), pair = (int)(i - (long)b * pairs);
+    float cs, sn;
+    rope_angle((float)positions[b], pair, head_dim, theta, cs, sn);
+    table[(long)b * head_dim + pair] = cs;
+    table[(long)b * head_dim + pairs + pair] = sn;
 }
 
 static int launch_rope(void *q_out, void *k_out, const void *q, const void *k,
@@ -177,6 +131,24 @@ static int launch_rope(void *q_out, void *k_out, const void *q, const void *k,
 }
 
 }  // namespace dskv
+
+extern "C" int dskv_rope_table(float *table, const int32_t *positions, int32_t batch,
+                               int32_t head_dim, float rope_theta, void *stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(batch >= 0, "rope_table: negative batch");
+    if (batch == 0) return 0;
+    DSKV_REQUIRE(table && positions, "rope_table: null pointer argument");
+    DSKV_REQUIRE(head_dim > 0 && head_dim % 8 == 0, "rope_table: head_dim %d must be a multiple of 8",
+                 head_dim);
+    DSKV_REQUIRE(rope_theta > 0.f, "rope_table: rope_theta must be positive");
+    DSKV_REQUIRE((uintptr_t)table % 16 == 0, "rope_table: the table must be 16-byte aligned");
+    const long n = (long)batch * (head_dim / 2);
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, table, positions, batch, head_dim, rope_theta);
+    DSKV_LAUNCH_CHECK("rope_table_kernel");
+    return 0;
+}
 
 extern "C" int dskv_apply_rope(void *q_out, void *k_out, const void *q, const void *k,
                                const int32_t *qo_indptr, const int32_t *offsets, int32_t batch,

@@ -29,10 +29,12 @@ class PagedAttentionCore:
         xk = xk.view(-1, self.n_local_kv_heads, self.head_dim)
         xv = xv.view(-1, self.n_local_kv_heads, self.head_dim)
         pages = ctx.page_pool.get_layered_pages(ctx.layer_id)
-        if (not self.use_rope and isinstance(ctx, FlashDecodeCtx) and self.fuse_decode_append
-                and xk.shape[0] == ctx.bsz and ctx.decode_wrapper.fused_append_supported(xq.dtype)):
-            # a decode step without rotation: the attention launch writes the new token itself
-            out = ctx.decode_wrapper.forward(xq, pages, k_append=xk, v_append=xv)
+        if (isinstance(ctx, FlashDecodeCtx) and self.fuse_decode_append and xk.shape[0] == ctx.bsz
+                and ctx.decode_wrapper.fused_append_supported(xq.dtype)):
+            # a decode step: the attention launch rotates q and the new k and writes the new
+            # token into its page slot itself
+            rope = dict(rope_offsets=ctx.offsets, rope_theta=self.rope_theta) if self.use_rope else {}
+            out = ctx.decode_wrapper.forward(xq, pages, k_append=xk, v_append=xv, **rope)
             return out.view(-1, self.dim)
         if self.use_rope and self.fuse_rope_append:
             # one kernel: rotated q comes back, rotated k and v go straight into their slots

@@ -94,6 +94,7 @@ class _PagedWrapper:
             raise ValueError("only the NHD page layout is implemented")
         self._workspace = workspace_buffer
         self._planned = False
+        self._rope_table, self._rope_key = None, None
 
     def _shape_args(self, num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> None:
         self._hq, self._hkv, self._d, self._p = num_qo_heads, num_kv_heads, head_dim, page_size
@@ -145,6 +146,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         if ws.value > self._workspace.numel() * self._workspace.element_size():
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
+        self._rope_table, self._rope_key = None, None     # positions change with the step
         if plan_buffers is not None:
             self._plan = plan_buffers.dev
             plan_buffers.upload(max(words.value, 1))
@@ -163,11 +165,16 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor,
                 sm_scale: Optional[float] = None, *, phases: int = 3,
                 out: Optional[torch.Tensor] = None, k_append: Optional[torch.Tensor] = None,
-                v_append: Optional[torch.Tensor] = None, **_ignored) -> torch.Tensor:
+                v_append: Optional[torch.Tensor] = None, rope_offsets: Optional[torch.Tensor] = None,
+                rope_theta: float = 500000.0, **_ignored) -> torch.Tensor:
         """phases: 1 = split-KV pass only, 2 = merge pass only, 3 = both (default).
         k_append, v_append (batch, Hkv, D): the step's token of every request, not yet in the
         pages - the attention launch writes them into their slots itself (one launch less than
-        append_paged_kv_cache + forward; see fused_append_supported)."""
+        append_paged_kv_cache + forward; see fused_append_supported).
+        rope_offsets (batch, int32, with k_append / v_append): the positions of those tokens;
+        q and k_append are then taken unrotated and rotated inside the launch (in place of
+        apply_rope before it).  The cos / sin table of the step is built at the first such call
+        after begin_forward and shared by the following layers."""
         if not self._planned:
             raise RuntimeError("decode forward called before begin_forward")
         q = q.contiguous()
@@ -187,6 +194,25 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
             if tuple(k_append.shape) != want or tuple(v_append.shape) != want or \
                     k_append.dtype != q.dtype or v_append.dtype != q.dtype:
                 raise ValueError(f"k_append / v_append must be {want} of q's dtype")
+            if rope_offsets is not None:
+                key = (rope_offsets.data_ptr(), float(rope_theta))
+                if self._rope_key != key:
+                    if rope_offsets.dtype != torch.int32 or rope_offsets.numel() != self._batch:
+                        raise ValueError(f"rope_offsets must be {self._batch} int32 positions")
+                    table = torch.empty((self._batch, self._d), dtype=torch.float32, device=q.device)
+                    _lib.check(_lib.lib().dskv_rope_table(table.data_ptr(), rope_offsets.data_ptr(),
+                                                          self._batch, self._d, rope_theta,
+                                                          _lib.current_stream()), "rope table")
+                    self._rope_table, self._rope_key = table, key
+                rc = _lib.lib().dskv_decode_rope_append_attn(
+                    out.data_ptr(), q.data_ptr(), k_append.data_ptr(), v_append.data_ptr(),
+                    paged_kv_data.data_ptr(), self._indices.data_ptr(), self._plan.data_ptr(),
+                    self._n_items, self._n_workgroups, self._workspace.data_ptr(), ws_bytes,
+                    self._batch, self._hq, self._hkv, self._d, self._p, scale,
+                    _lib.dtype_code(q.dtype), self._rope_table.data_ptr(), phases,
+                    _lib.current_stream())
+                _lib.check(rc, "decode rope + append + forward")
+                return out
             rc = _lib.lib().dskv_decode_append_attn(
                 out.data_ptr(), q.data_ptr(), k_append.data_ptr(), v_append.data_ptr(),
                 paged_kv_data.data_ptr(), self._indices.data_ptr(), self._plan.data_ptr(),

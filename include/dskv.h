@@ -145,6 +145,27 @@ int dskv_decode_append_attn(void *out, const void *q, const void *k_new, const v
                             void *stream);
 
 /*
+ * The same with the rotary embedding of the step inside the launch: q is
+ * rotated as it is loaded and k_new before it is stored, with the adjacent-pair
+ * convention and arithmetic of dskv_apply_rope, so a decode step of a layer is
+ * this one launch (plus the merge pass) in place of
+ * apply_rope + append_paged_kv_cache + forward (model/layer/attention.py:166-187).
+ * rope_table: (batch, head_dim) floats, row b = cos | sin of
+ * positions[b] * theta^(-2*pair/head_dim) for the head_dim/2 pairs, written by
+ * dskv_rope_table from the device array of the new tokens' positions (the
+ * reference's ctx.offsets); built once per step, shared by all layers.
+ */
+int dskv_rope_table(float *table, const int32_t *positions, int32_t batch, int32_t head_dim,
+                    float rope_theta, void *stream);
+int dskv_decode_rope_append_attn(void *out, const void *q, const void *k_new, const void *v_new,
+                                 void *pages_layer, const int32_t *kv_page_indices,
+                                 const int32_t *plan_dev, int32_t n_items, int32_t n_workgroups,
+                                 void *workspace, int64_t workspace_bytes, int32_t batch,
+                                 int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                                 int32_t page_size, float sm_scale, int32_t dtype,
+                                 const float *rope_table, int32_t phases, void *stream);
+
+/*
  * Paged prefill attention with the end-aligned causal mask.  Replaces
  * BatchPrefillWithPagedKVCacheWrapper.forward(q, pages, causal=True)
  * (model/layer/attention.py:188-192, execution/exec.py:227-236).

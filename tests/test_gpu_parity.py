@@ -357,6 +357,43 @@ def test_decode_with_fused_append_equals_append_then_decode(case):
     w.end_forward()
 
 
+@pytest.mark.parametrize("case", FUSED_CASES, ids=[c[0] for c in FUSED_CASES])
+def test_decode_with_rope_inside_equals_rope_append_then_decode(case):
+    """forward(k_append=, v_append=, rope_offsets=) against rope_append_paged_kv_cache + forward:
+    the same pages and the same output, bit for bit (one rotation arithmetic, shared), and both
+    within tolerance of the oracle's rotation + append + attention."""
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper, rope_append_paged_kv_cache
+
+    name, kv, P, Hq, Hkv, D, dtype, target = case
+    _announce("decode fused rope", name)
+    sc = make_scenario(913, kv_lens=kv, qo_lens=[1] * len(kv), P=P, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype)
+    offsets = (np.asarray(kv, np.int64) - 1).astype(np.int32)            # position of the new token
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
+    meta = (_dev_i32(sc.kv_page_indices), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_last_page_lens))
+    w.begin_forward(meta[1], meta[0], meta[2], Hq, Hkv, D, P, target_workgroups=target)
+    q, k, v = to_torch(sc.q, dtype), to_torch(sc.k, dtype), to_torch(sc.v, dtype)
+    pages_a, pages_b = to_torch(sc.pages, dtype), to_torch(sc.pages, dtype)
+    q_rot = rope_append_paged_kv_cache(q, k, v, _dev_i32(sc.qo_indptr), _dev_i32(offsets), pages_a, *meta,
+                                       rope_theta=5e5)
+    out_a = w.forward(q_rot, pages_a)
+    out_b = w.forward(q, pages_b, k_append=k, v_append=v, rope_offsets=_dev_i32(offsets), rope_theta=5e5)
+    torch.cuda.synchronize()
+    assert _same_bits(from_torch(pages_b, dtype), from_torch(pages_a, dtype))
+    assert _same_bits(from_torch(out_b, dtype), from_torch(out_a, dtype))
+    # against the oracle: rotate, append, attend in fp32
+    q32, k32 = orc.to_f32(sc.q, dtype), orc.to_f32(sc.k, dtype)
+    q_ref = orc.rope_interleaved(q32, sc.qo_indptr, offsets)
+    k_ref = orc.rope_interleaved(k32, sc.qo_indptr, offsets)
+    from kvutil import to_storage
+    want_pages = sc.pages.copy()
+    orc.append_paged_kv(want_pages, to_storage(k_ref, dtype), sc.v, sc.qo_indptr, sc.kv_page_indices,
+                        sc.kv_page_indptr, sc.kv_last_page_lens)
+    want = c_oracle.decode_attn(to_storage(q_ref, dtype), want_pages, sc.kv_page_indices,
+                                sc.kv_page_indptr, sc.kv_last_page_lens, dtype)
+    assert max_rel_err(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
+    w.end_forward()
+
+
 def test_fused_append_is_refused_outside_the_mfma_shapes():
     from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
 
