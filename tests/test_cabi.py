@@ -56,6 +56,12 @@ def test_argument_errors_return_negative_codes_without_a_gpu():
     assert lib.dskv_decode_append_attn(16, 16, 16, 24, *fused[4:], 2, 3, None) == -1 and "aligned" in _lib.last_error()
     assert lib.dskv_decode_append_attn(*fused, 0, 3, None) == -1 and "separately" in _lib.last_error()   # fp32
     assert lib.dskv_decode_append_attn(*fused[:11], 0, *fused[12:], 2, 3, None) == 0                    # empty batch
+    assert lib.dskv_decode_rope_append_attn(*fused, 2, None, 3, None) == -1 and "table" in _lib.last_error()
+    assert lib.dskv_decode_rope_append_attn(*fused, 2, 16, 2, None) == -1 and "phases" in _lib.last_error()
+    assert lib.dskv_decode_rope_append_attn(*fused, 0, 16, 3, None) == -1 and "separately" in _lib.last_error()
+    assert lib.dskv_rope_table(16, 16, -1, 128, 5e5, None) == -1 and lib.dskv_rope_table(None, None, 0, 128, 5e5, None) == 0
+    assert lib.dskv_rope_table(16, 16, 2, 100, 5e5, None) == -1 and lib.dskv_rope_table(16, 16, 2, 128, 0.0, None) == -1
+    assert lib.dskv_rope_table(8, 16, 2, 128, 5e5, None) == -1 and "aligned" in _lib.last_error()
     assert lib.dskv_decode_append_attn_supported(32, 8, 128, 16, 2) == 1
     assert lib.dskv_decode_append_attn_supported(32, 8, 128, 16, 0) == 0      # fp32 pool
     assert lib.dskv_decode_append_attn_supported(32, 8, 64, 16, 2) == 0       # head_dim
