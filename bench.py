@@ -465,7 +465,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     L, Hq, Hkv, D, P = 16, 32, 8, 128, 16
     graph_steps = 0 if a.no_graph else 24
-    total_steps = a.steps + a.warmup + graph_steps
+    rope_steps = 0 if a.rope else 24          # the step once more with rotation, as a model runs it
+    total_steps = a.steps + a.warmup + graph_steps + rope_steps
     ctx = config2_context_lengths(a.seed)
     wl = make_decode_workload("cfg2", ctx, L, Hq, Hkv, D, P, torch.bfloat16,
                               headroom_tokens=total_steps + 8, seed=a.seed, use_rope=a.rope)
@@ -496,7 +497,7 @@ def main() -> int:
 
     fused = not a.no_fused_append
 
-    def one_step(timed: bool):
+    def one_step(timed: bool, rope: bool = a.rope):
         """prepare (metadata + plan, one upload each) then L x (append + attention: one launch
         for both, or two with --no-fused-append)."""
         c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, decode_wrapper)
@@ -512,11 +513,11 @@ def main() -> int:
             if fused:
                 # the attention launch (rotates q and k and) writes the token
                 new_kv = dict(k_append=k, v_append=v)
-                if a.rope:
+                if rope:
                     new_kv.update(rope_offsets=c.offsets, rope_theta=5e5)
             else:
                 new_kv = {}
-                if a.rope:
+                if rope:
                     q = rope_append_paged_kv_cache(q, k, v, c.indptr, c.offsets, pages, c.kv_page_indices,
                                                    c.kv_page_indptr, c.kv_last_page_lens, rope_theta=5e5)
                 else:
@@ -569,6 +570,19 @@ def main() -> int:
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     loop_ms = np.diff(np.array(marks)) * 1e3       # host time per loop turn (enqueue + its wait)
+    rope_ms = None
+    if rope_steps:
+        for _ in range(4):
+            one_step(False, rope=True)
+        torch.cuda.synchronize()
+        r0 = time.perf_counter()
+        for i in range(rope_steps - 4):
+            ev = wait_turn(i)
+            one_step(False, rope=True)
+            if ev is not None:
+                ev.record()
+        torch.cuda.synchronize()
+        rope_ms = (time.perf_counter() - r0) / (rope_steps - 4) * 1e3
 
     ms_per_step = elapsed / a.steps * 1e3
     value = sum(step_bytes) / elapsed / 1e9
@@ -586,6 +600,7 @@ def main() -> int:
                    "append": "inside the attention launch" if fused else "own launch"},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "stage_tokens_per_s": round(wl.batch / (elapsed / a.steps), 1),
+        "with_rope_ms_per_step": None if rope_ms is None else round(rope_ms, 4),
         "host_loop_ms": {"median": round(float(np.median(loop_ms)), 3), "max": round(float(loop_ms.max()), 3),
                          "turns_over_3ms": int((loop_ms > 3.0).sum())},
     }
