@@ -87,7 +87,7 @@ def test_gather_scatter_bit_exact(dtype, P):
         if ids:
             assert _same_bits(c_oracle.gather(host, ids), want)
     ids = [9, 2, 30]
-    chunk = rng.integers(0, 2**16, size=(L * 3,) + host.shape[2:]).astype(host.dtype) \
+    chunk = rng.integers(0, 2**16, size=(L * 3,) + host.shape[2:], dtype=np.uint16).view(host.dtype) \
         if dtype != "f32" else rng.standard_normal((L * 3,) + host.shape[2:]).astype(np.float32)
     want = host.copy()
     orc.scatter_pages(want, ids, chunk)
