@@ -58,6 +58,7 @@ def parse_args():
     ap.add_argument("--steps-in-flight", type=int, default=2,
                     help="steps the host may have queued on the GPU (a stage hands every step's "
                          "output on before it starts the next but one); 0 = no limit")
+    ap.add_argument("--no-rope-step", action="store_true", help="skip the extra steps with rotation")
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--section", choices=["swap", "fragmented", "prefill"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
@@ -465,7 +466,7 @@ def main() -> int:
     torch.cuda.set_device(0)
     L, Hq, Hkv, D, P = 16, 32, 8, 128, 16
     graph_steps = 0 if a.no_graph else 24
-    rope_steps = 0 if a.rope else 24          # the step once more with rotation, as a model runs it
+    rope_steps = 0 if (a.rope or a.no_rope_step) else 24          # the step once more with rotation, as a model runs it
     total_steps = a.steps + a.warmup + graph_steps + rope_steps
     ctx = config2_context_lengths(a.seed)
     wl = make_decode_workload("cfg2", ctx, L, Hq, Hkv, D, P, torch.bfloat16,
