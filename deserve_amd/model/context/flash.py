@@ -34,28 +34,49 @@ _FIELDS = ("indptr", "kv_page_indptr", "kv_last_page_lens", "offsets", "seqlens"
 
 def build_host_metadata(task_datas: Sequence[TaskData],
                         kvcaches: Sequence[PagedKVCache]) -> Dict[str, np.ndarray]:
-    """The six int32 arrays on the host; extends the caches as a side effect."""
+    """The six int32 arrays on the host; extends the caches as a side effect (in request
+    order, as the reference's loop does: the order decides which page ids a request gets)."""
     B = len(task_datas)
+    start = np.fromiter((t.start_pos for t in task_datas), np.int64, B)
+    seq = np.fromiter((t.seqlen for t in task_datas), np.int64, B)
+    want = np.fromiter((t.initial_seqlen for t in task_datas), np.int64, B)
+    current = start + seq
+    np.maximum(want, current, out=want)
     indptr = np.zeros(B + 1, np.int32)
+    np.cumsum(seq, out=indptr[1:])
+    one_pool = B > 0 and all(c.pool is kvcaches[0].pool for c in kvcaches)
+    one_table = one_pool and all(c.page_table.allocator is kvcaches[0].page_table.allocator
+                                 for c in kvcaches)
+    if not one_table:
+        # caches over several pools or tables: request by request
+        exposed = np.zeros(B, np.int64)
+        last = np.zeros(B, np.int32)
+        rows: List[np.ndarray] = []
+        for i, cache in enumerate(kvcaches):
+            page_size = cache.pool.page_size
+            cache.extend(int(want[i]))
+            exposed[i] = -(-int(current[i]) // page_size)
+            rows.append(cache.page_table.retrieve()[: int(exposed[i])].numpy())
+            last[i] = (int(current[i]) - 1) % page_size + 1
+        indices = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
+    else:
+        # the usual case, without a Python-level pass per request: only the caches that
+        # cross a page boundary are touched, and the block-table rows are gathered at once
+        page_size = kvcaches[0].pool.page_size
+        have = np.fromiter((c.page_table.occupied for c in kvcaches), np.int64, B) * page_size
+        for i in np.flatnonzero(want > have):
+            kvcaches[i].extend(int(want[i]))
+        exposed = -(-current // page_size)
+        last = ((current - 1) % page_size + 1).astype(np.int32)
+        table = kvcaches[0].page_table.allocator.tables.numpy()
+        slots = np.fromiter((c.page_table.offset for c in kvcaches), np.int64, B)
+        width = int(exposed.max())
+        picked = table[slots, :width]
+        indices = picked[np.arange(width)[None, :] < exposed[:, None]].astype(np.int32, copy=False)
     kv_indptr = np.zeros(B + 1, np.int32)
-    last = np.zeros(B, np.int32)
-    offsets = np.zeros(B, np.int32)
-    seqlens = np.zeros(B, np.int32)
-    rows: List[np.ndarray] = []
-    for i, (task, cache) in enumerate(zip(task_datas, kvcaches)):
-        page_size = cache.pool.page_size
-        current_len = task.start_pos + task.seqlen
-        cache.extend(max(current_len, task.initial_seqlen))
-        exposed = -(-current_len // page_size)
-        rows.append(cache.page_table.retrieve()[:exposed].numpy())
-        last[i] = (current_len - 1) % page_size + 1
-        offsets[i] = task.start_pos
-        seqlens[i] = task.seqlen
-        indptr[i + 1] = indptr[i] + task.seqlen
-        kv_indptr[i + 1] = kv_indptr[i] + exposed
-    indices = np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
-    return dict(indptr=indptr, kv_page_indptr=kv_indptr, kv_last_page_lens=last, offsets=offsets,
-                seqlens=seqlens, kv_page_indices=indices)
+    np.cumsum(exposed, out=kv_indptr[1:])
+    return dict(indptr=indptr, kv_page_indptr=kv_indptr, kv_last_page_lens=last,
+                offsets=start.astype(np.int32), seqlens=seq.astype(np.int32), kv_page_indices=indices)
 
 
 class StagedUpload:
