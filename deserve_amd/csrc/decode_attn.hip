@@ -288,7 +288,9 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
         for (int t = item.tok_begin; t < t_pad_end; t += kStages * kTile) {
 #pragma unroll
             for (int s = 0; s < kStages; s++) {
-                compute_tile(t + s * kTile, ring[s]);
+                // a padding tile (items are padded to whole rounds of the ring) holds nothing:
+                // its loads were issued and fetched nothing, its work is skipped (wave-uniform)
+                if (t + s * kTile < t_end) compute_tile(t + s * kTile, ring[s]);
                 // keep the scheduler from hoisting a later tile's work (and its
                 // wait for younger loads) above this point
                 __builtin_amdgcn_sched_barrier(0);
