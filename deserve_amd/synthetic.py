@@ -8,7 +8,7 @@ records at the given context lengths, and per-layer q/k/v inputs ~ N(0, 1).
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Optional, Sequence
+from typing import List, Sequence
 
 import numpy as np
 import torch

@@ -8,9 +8,9 @@ import numpy as np
 import pytest
 import torch
 
-from kvutil import from_torch, max_rel_err
+from kvutil import max_rel_err
 from oracle import c_oracle
-from oracle import kv_oracle as orc
+
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda")

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from kvutil import from_torch, max_rel_err, to_storage
+from kvutil import max_rel_err
 from oracle import kv_oracle as orc
 
 pytestmark = pytest.mark.gpu

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 from scipy.special import softmax
 
-from kvutil import make_scenario, max_rel_err, to_storage
+from kvutil import make_scenario
 from oracle import c_oracle
 from oracle import kv_oracle as orc
 
