@@ -124,6 +124,8 @@ DECODE_CASES = [
     ("mha", [300, 40], 16, 8, 8, 128, "bf16", 0),
     ("group16", [300, 40], 16, 32, 2, 128, "bf16", 8),
     ("kv4", [300, 40, 1], 16, 16, 4, 128, "bf16", 0),
+    ("kv16", [300, 40, 17, 1000], 16, 32, 16, 128, "bf16", 12),    # two groups of 8 kv heads per workgroup id
+    ("kv12", [200, 33], 16, 24, 12, 128, "f16", 0),                # the second group half full
     ("f32", [512, 100, 1, 33], 16, 32, 8, 128, "f32", 8),
     ("f32_d64", [200, 17], 8, 8, 2, 64, "f32", 0),
     ("bf16_d64_generic", [200, 17], 16, 8, 2, 64, "bf16", 4),
