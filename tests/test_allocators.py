@@ -340,3 +340,31 @@ def test_task_manager_page_arithmetic():
     a.step()
     assert (a.start_pos, a.seqlen, a.round) == (20, 1, 1) and a.is_prefill()
     assert tm.calc_delta_space("a", 1) == 0 and tm.calc_occupied_space(["a"]) == 3
+
+
+def test_ctx_builder_empty_batch_and_caches_over_two_pools():
+    """The builder's two routes (block-table rows gathered at once / request by request for
+    caches that do not share one pool and table) give the same arrays."""
+    meta = build_host_metadata([], [])
+    assert meta["indptr"].tolist() == [0] and meta["kv_page_indptr"].tolist() == [0]
+    assert all(meta[k].shape == (0,) for k in ("kv_last_page_lens", "offsets", "seqlens", "kv_page_indices"))
+    P = 8
+    lens = [5, 8, 9, 40]
+
+    def build(pools, tables):
+        tasks, caches = [], []
+        for i, n in enumerate(lens):
+            tasks.append(TaskData(f"t{i}", n - 1, 1, 1, n - 1, SamplingParams()))
+            caches.append(PagedKVCache.empty(tables[i % len(tables)], pools[i % len(pools)]))
+        return build_host_metadata(tasks, caches), caches
+
+    one, caches_one = build([CpuPagePool(1, 64, P, torch.float32, 1, 1)], [PageTableAllocator(8, 256, P, CPU)])
+    two, caches_two = build([CpuPagePool(1, 64, P, torch.float32, 1, 1), CpuPagePool(1, 64, P, torch.float32, 1, 1)],
+                            [PageTableAllocator(8, 256, P, CPU), PageTableAllocator(8, 256, P, CPU)])
+    for k in ("indptr", "kv_page_indptr", "kv_last_page_lens", "offsets", "seqlens"):
+        assert np.array_equal(one[k], two[k]), k
+    assert one["kv_page_indptr"].tolist() == [0, 1, 2, 4, 9] and one["kv_last_page_lens"].tolist() == [5, 8, 1, 8]
+    # page ids: one pool hands them out in request order; with two pools each pool does
+    assert one["kv_page_indices"].tolist() == list(range(9))
+    assert two["kv_page_indices"].tolist() == [0, 0, 1, 2, 1, 2, 3, 4, 5]
+    assert [c.page_table.occupied for c in caches_one] == [1, 1, 2, 5]
