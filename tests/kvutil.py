@@ -82,6 +82,22 @@ def max_rel_err(got: np.ndarray, ref: np.ndarray) -> float:
                  max(float(np.abs(ref).max()), 1e-30))
 
 
+def max_rel_err_per_request(got: np.ndarray, ref: np.ndarray, row_indptr=None) -> float:
+    """The largest max_rel_err over requests, each request measured against the scale of
+    its OWN output: a long request's output is a mean over thousands of values and far
+    smaller than a short one's, so a scale taken over the whole batch would let any error
+    in it pass.  row_indptr: CSR bounds of every request's block of rows along axis 0
+    (prefill); None = one row per request (decode).  Requests without rows are skipped."""
+    if row_indptr is None:
+        row_indptr = np.arange(got.shape[0] + 1)
+    worst = 0.0
+    for b in range(len(row_indptr) - 1):
+        lo, hi = int(row_indptr[b]), int(row_indptr[b + 1])
+        if hi > lo:
+            worst = max(worst, max_rel_err(got[lo:hi], ref[lo:hi]))
+    return worst
+
+
 # ---- torch <-> storage helpers (GPU tests only)
 def torch_dtype(dtype: str):
     import torch

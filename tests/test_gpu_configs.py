@@ -8,8 +8,9 @@ import numpy as np
 import pytest
 import torch
 
-from kvutil import max_rel_err
+from kvutil import max_rel_err_per_request
 from oracle import c_oracle
+from oracle import kv_oracle as orc
 
 
 pytestmark = pytest.mark.gpu
@@ -29,8 +30,10 @@ def _bits(t: torch.Tensor) -> np.ndarray:
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
-def _decode_step(wl, wrapper, layers, rope=False):
-    """One engine-style decode step over the given layers; returns (ctx, {layer: out})."""
+def _decode_step(wl, wrapper, layers, fused=False, rope=False):
+    """One engine-style decode step over the given layers; returns (ctx, {layer: out}).
+    fused: the attention launch writes the step's token itself (the form the bench times);
+    rope (with fused): it also rotates q and the new k at the tokens' positions."""
     from deserve_amd.model.context.flash import FlashDecodeCtx
     from deserve_amd.paged_ops import append_paged_kv_cache
 
@@ -44,27 +47,35 @@ def _decode_step(wl, wrapper, layers, rope=False):
     outs = {}
     for layer in layers:
         pages = wl.pool.get_layered_pages(layer)
-        append_paged_kv_cache(wl.k[layer], wl.v[layer], ctx.indptr, pages, ctx.kv_page_indices,
-                              ctx.kv_page_indptr, ctx.kv_last_page_lens)
-        outs[layer] = wrapper.forward(wl.q[layer], pages)
+        if fused:
+            extra = dict(rope_offsets=ctx.offsets, rope_theta=5e5) if rope else {}
+            outs[layer] = wrapper.forward(wl.q[layer], pages, k_append=wl.k[layer], v_append=wl.v[layer],
+                                          **extra)
+        else:
+            append_paged_kv_cache(wl.k[layer], wl.v[layer], ctx.indptr, pages, ctx.kv_page_indices,
+                                  ctx.kv_page_indptr, ctx.kv_last_page_lens)
+            outs[layer] = wrapper.forward(wl.q[layer], pages)
+    plan_shape = (wrapper._n_items, wrapper._n_workgroups)
     wrapper.end_forward()
     torch.cuda.synchronize()
-    return ctx, outs
+    return ctx, outs, plan_shape
 
 
-def _oracle_rows(wl, ctx, layer, requests):
-    """fp32 oracle output for a sample of requests: their pages are copied to the host."""
-    P = wl.args.page_size
+def _oracle_rows(wl, ctx, layer, requests, q_bits=None):
+    """fp32 oracle output (C port, fp32 accumulation) of the given requests, in their order:
+    their pages are copied to the host as one compact array and attended in one call.
+    q_bits: (B, Hq, D) bf16 bit patterns to use instead of the workload's q of the layer."""
     indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
     last = ctx.host["kv_last_page_lens"].numpy()
-    want = {}
-    for b in requests:
-        ids = ids_all[indptr[b]: indptr[b + 1]]
-        pages = _bits(wl.pool.pages[layer].index_select(0, torch.from_numpy(ids.astype(np.int64)).to(DEV)))
-        q = _bits(wl.q[layer, b: b + 1])
-        want[b] = c_oracle.decode_attn(q, pages, np.arange(len(ids), dtype=np.int32),
-                                       np.array([0, len(ids)], np.int32), last[b: b + 1], "bf16")[0]
-    return want
+    requests = np.asarray(list(requests), dtype=np.int64)
+    ids = np.concatenate([ids_all[indptr[b]: indptr[b + 1]] for b in requests])
+    local_indptr = np.concatenate([[0], np.cumsum(indptr[requests + 1] - indptr[requests])]).astype(np.int32)
+    pages = _bits(wl.pool.pages[layer].index_select(0, torch.from_numpy(ids.astype(np.int64)).to(DEV)))
+    if q_bits is None:
+        q_bits = _bits(wl.q[layer])
+    return c_oracle.decode_attn(np.ascontiguousarray(q_bits[requests]), pages,
+                                np.arange(len(ids), dtype=np.int32), local_indptr,
+                                np.ascontiguousarray(last[requests]), "bf16")
 
 
 def _check_append(wl, ctx, layer, before_sum, old_rows):
@@ -95,37 +106,85 @@ def _old_rows_sum(wl, layer):
     return _checksum(rows)
 
 
+def _check_rope_append(wl, ctx, layer, before_sum, old_rows):
+    """After the launch that rotates and appends: the new V rows equal v bit for bit, the new
+    K rows are the oracle's rotation of k at the tokens' positions to within one bf16 ulp, and
+    the checksum of the layer moved by exactly (new rows - old rows).  Returns the K rows as
+    the device wrote them."""
+    indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
+    last = ctx.host["kv_last_page_lens"].numpy()
+    page = torch.from_numpy(ids_all[indptr[1:] - 1].astype(np.int64)).to(DEV)
+    slot = torch.from_numpy((last - 1).astype(np.int64)).to(DEV)
+    got = wl.pool.pages[layer][page, :, slot]                       # (B, 2, Hkv, D)
+    assert torch.equal(got[:, 1].view(torch.int16), wl.v[layer].view(torch.int16))
+    k_ref = orc.rope_interleaved(orc.f32_from_bf16_bits(_bits(wl.k[layer])), ctx.host["indptr"].numpy(),
+                                 ctx.host["offsets"].numpy())
+    k_dev = orc.f32_from_bf16_bits(_bits(got[:, 0]))
+    assert np.abs(k_dev - k_ref).max() <= 2.0 ** -7 * max(float(np.abs(k_ref).max()), 1.0)
+    delta = _checksum(got) - old_rows
+    assert _checksum(wl.pool.pages[layer]) == before_sum + delta, "bytes outside the new rows changed"
+
+
 def test_config2_llama8b_stage_decode_step_full_size():
+    """The step the bench times: the attention launch of every layer writes the step's token
+    itself, with the default plan (one persistent workgroup per CU, most requests cut).  Pages
+    against the append's definition bit for bit; ALL 64 requests of three layers against the
+    C oracle, each request against its own output scale.  Then the same with the rotation
+    inside the launch on two more layers, and the append-then-attend pair on relocated pages."""
     from deserve_amd.execution.exec import get_wrappers
     from deserve_amd.synthetic import config2_context_lengths, make_decode_workload
 
-    _announce("config2 full size")
+    _announce("config2 full size, fused append")
     wl = make_decode_workload("cfg2", config2_context_lengths(2), 16, 32, 8, 128, 16, torch.bfloat16,
                               headroom_tokens=32, seed=2)
     wrapper, _ = get_wrappers(DEV)
+    B = wl.batch
     layers = [0, 7, 15]
     before = {l: _checksum(wl.pool.pages[l]) for l in layers}
     old = {l: _old_rows_sum(wl, l) for l in layers}
-    ctx, outs = _decode_step(wl, wrapper, layers)
-    sample = [int(np.argmax(wl.ctx_lens)), int(np.argmin(wl.ctx_lens)), 5]
+    ctx, outs, (n_items, n_wgs) = _decode_step(wl, wrapper, layers, fused=True)
+    assert n_wgs == torch.cuda.get_device_properties(0).multi_processor_count
+    assert n_items > B                                      # the plan of the bench: requests are cut
     for l in layers:
         _check_append(wl, ctx, l, before[l], old[l])
-    want = _oracle_rows(wl, ctx, 7, sample)
-    got = outs[7].float().cpu().numpy()
-    for b in sample:
-        assert max_rel_err(got[b], want[b]) <= 2e-2, b
-    assert torch.isfinite(outs[0].float()).all() and torch.isfinite(outs[15].float()).all()
-    # relocating every page of the layer (and renaming it in the block table) changes nothing
+        want = _oracle_rows(wl, ctx, l, range(B))
+        got = outs[l].float().cpu().numpy()
+        assert np.isfinite(got).all()
+        err = max_rel_err_per_request(got, want)
+        _announce("config2 layer", l, "worst request error", err)
+        assert err <= 2e-2, l
+    # append-then-attend on the same pages gives the same bits (the token is there already),
+    # also after relocating every page of the layer and renaming it in the block table
     perm = torch.randperm(wl.pool.num_pages, device=DEV)
     moved = torch.empty_like(wl.pool.pages[7])
     moved[perm] = wl.pool.pages[7]
     new_ids = perm[ctx.kv_page_indices.long()].to(torch.int32)
-    wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=new_ids, last_page_len=ctx.kv_last_page_lens,
-                          num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
-                          indptr_host=ctx.host["kv_page_indptr"], last_page_len_host=ctx.host["kv_last_page_lens"])
-    again = wrapper.forward(wl.q[7], moved)
-    wrapper.end_forward()
-    assert torch.equal(again.view(torch.int16), outs[7].view(torch.int16))
+    for ids, pages in ((ctx.kv_page_indices, wl.pool.pages[7]), (new_ids, moved)):
+        wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ids, last_page_len=ctx.kv_last_page_lens,
+                              num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
+                              indptr_host=ctx.host["kv_page_indptr"],
+                              last_page_len_host=ctx.host["kv_last_page_lens"])
+        again = wrapper.forward(wl.q[7], pages)
+        wrapper.end_forward()
+        assert torch.equal(again.view(torch.int16), outs[7].view(torch.int16))
+    del moved
+
+    _announce("config2 full size, rotation + append inside the launch")
+    for t in wl.tasks:
+        t.step()
+    layers = [3, 12]
+    before = {l: _checksum(wl.pool.pages[l]) for l in layers}
+    old = {l: _old_rows_sum(wl, l) for l in layers}
+    ctx, outs, _ = _decode_step(wl, wrapper, layers, fused=True, rope=True)
+    for l in layers:
+        _check_rope_append(wl, ctx, l, before[l], old[l])
+        q_rot = orc.rope_interleaved(orc.f32_from_bf16_bits(_bits(wl.q[l])), ctx.host["indptr"].numpy(),
+                                     ctx.host["offsets"].numpy())
+        want = _oracle_rows(wl, ctx, l, range(B), q_bits=orc.bf16_bits_from_f32(q_rot))
+        got = outs[l].float().cpu().numpy()
+        err = max_rel_err_per_request(got, want)
+        _announce("config2 layer", l, "worst request error with rotation", err)
+        assert np.isfinite(got).all() and err <= 2e-2, l
 
 
 def test_config3_microbatch_exchange_round_trip_full_size():
@@ -163,7 +222,7 @@ def test_config3_microbatch_exchange_round_trip_full_size():
     eng.close()
 
 
-def test_config4_chunked_prefill_full_batch_two_layers():
+def test_config4_chunked_prefill_full_batch_four_layers():
     """16 sequences append a 512-token chunk behind a prior of U[0, 8192] tokens that ends
     mid-page (offset U[0, 15]), then attend causally over prior + chunk."""
     from deserve_amd.kvcache.paged.kvcache import PagedKVCache
@@ -175,7 +234,7 @@ def test_config4_chunked_prefill_full_batch_two_layers():
     from deserve_amd.task import SamplingParams, TaskData
 
     _announce("config4")
-    L, P, Hq, Hkv, D, B, n = 2, 16, 32, 8, 128, 16, 512
+    L, P, Hq, Hkv, D, B, n = 4, 16, 32, 8, 128, 16, 512
     rng = np.random.default_rng(4)
     prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
     prior[0], prior[1] = 0, 8192 + 15                               # extremes: pure prompt, longest
@@ -216,20 +275,38 @@ def test_config4_chunked_prefill_full_batch_two_layers():
         outs.append(w.forward(q[l], pool.pages[l], causal=True))
     torch.cuda.synchronize()
     w.end_forward()
-    # oracle on sampled query rows: row i of request b is decode attention over prior_b + i + 1 tokens
-    layer = 1
-    got = outs[layer].float().cpu().numpy()
-    for b, i in [(0, 0), (0, 511), (1, 0), (1, 300), (1, 511), (7, 17), (15, 256)]:
-        limit = int(prior[b]) + i + 1
-        npg = -(-limit // P)
-        ids = ids_all[indptr[b]: indptr[b] + npg]
+    # oracle on sampled query rows: row i of request b is decode attention over
+    # prior_b + i + 1 tokens.  Per layer 16 rows: first and last row of the shortest and of
+    # the longest prior (requests 0 and 1), a row that ends on a page boundary, and seeded ones
+    # over all requests; every row against its own output scale.
+    worst = 0.0
+    for layer in range(L):
+        picks = [(0, 0), (0, n - 1), (1, 0), (1, n - 1), (2, int((-prior[2] - 1) % P))]
+        picks += [(int(rng.integers(0, B)), int(rng.integers(0, n))) for _ in range(11)]
+        reqs = sorted({b for b, _ in picks})
+        base, run = {}, 0
+        for b in reqs:
+            base[b] = run
+            run += int(indptr[b + 1] - indptr[b])
+        ids = np.concatenate([ids_all[indptr[b]: indptr[b + 1]] for b in reqs])
         pages = _bits(pool.pages[layer].index_select(0, torch.from_numpy(ids.astype(np.int64)).to(DEV)))
-        row = b * n + i
-        want = c_oracle.decode_attn(_bits(q[layer, row: row + 1]), pages, np.arange(npg, dtype=np.int32),
-                                    np.array([0, npg], np.int32),
-                                    np.array([(limit - 1) % P + 1], np.int32), "bf16")[0]
-        assert max_rel_err(got[row], want) <= 2e-2, (b, i)
-    assert np.isfinite(got).all()
+        tables, counts, lasts, rows_q = [], [], [], []
+        for b, i in picks:
+            limit = int(prior[b]) + i + 1
+            npg = -(-limit // P)
+            tables.append(base[b] + np.arange(npg, dtype=np.int32))
+            counts.append(npg)
+            lasts.append((limit - 1) % P + 1)
+            rows_q.append(b * n + i)
+        want = c_oracle.decode_attn(np.ascontiguousarray(_bits(q[layer])[rows_q]), pages,
+                                    np.concatenate(tables), np.concatenate([[0], np.cumsum(counts)]),
+                                    np.asarray(lasts), "bf16")
+        got = outs[layer].float().cpu().numpy()
+        assert np.isfinite(got).all()
+        err = max_rel_err_per_request(got[rows_q], want)
+        worst = max(worst, err)
+        assert err <= 2e-2, (layer, picks)
+    _announce("config4 worst sampled row error", worst)
 
 
 def test_config5_fragmented_pool_swap_in_then_decode():
@@ -249,6 +326,7 @@ def test_config5_fragmented_pool_swap_in_then_decode():
     L, P, Hq, Hkv, D, B = 10, 16, 64, 8, 128, 128
     rng = np.random.default_rng(5)
     ctx_lens = config5_context_lengths(5)
+    ctx_lens[np.argmax(ctx_lens)], ctx_lens[np.argmin(ctx_lens)] = 32768, 64      # both clip bounds occur
     need = int((-(-(ctx_lens + 8) // P)).sum())
     pool = VirtualPagePool(L, int(need / 0.4 * 1.05) + 128, 0, P, DEV, torch.bfloat16)   # 40 % of it must hold everything
     fill_normal(pool.pages, 8)
@@ -270,7 +348,7 @@ def test_config5_fragmented_pool_swap_in_then_decode():
         caches.append(made[b])
     ids0 = caches[0].page_table.retrieve().numpy()
     assert np.any(np.diff(ids0) != 1), "block table should be fragmented"
-    mgr = KVCacheManager(pool, CpuChunkPool(L, 14, P, torch.bfloat16), rows)
+    mgr = KVCacheManager(pool, CpuChunkPool(L, 15, P, torch.bfloat16), rows)
     swapped = sorted(rng.choice(B, size=B // 4, replace=False).tolist())
     images = {b: pool.retrieve(caches[b].page_table.retrieve()) for b in swapped[:4]}
     handles = [mgr.copy_gpu_to_cpu(caches[b], tasks[b].task_id) for b in swapped]
@@ -292,13 +370,22 @@ def test_config5_fragmented_pool_swap_in_then_decode():
     wl = DecodeWorkload("cfg5", args, pool, rows, tasks, caches, KVStage(args, use_rope=False),
                         mk(Hq), mk(Hkv), mk(Hkv), ctx_lens)
     wrapper, _ = get_wrappers(DEV)
-    layer = 4
-    before, old = _checksum(pool.pages[layer]), _old_rows_sum(wl, layer)
-    ctx, outs = _decode_step(wl, wrapper, [layer])
-    _check_append(wl, ctx, layer, before, old)
-    sample = [int(np.argmax(ctx_lens)), int(np.argmin(ctx_lens)), swapped[0], swapped[-1]]
-    want = _oracle_rows(wl, ctx, layer, sample)
-    got = outs[layer].float().cpu().numpy()
-    for b in sample:
-        assert max_rel_err(got[b], want[b]) <= 2e-2, b
-    assert np.isfinite(got).all()
+    # 16 requests against the oracle: the longest (32 k tokens, cut into dozens of parts), the
+    # shortest, four of the swapped ones and seeded others; one layer with the append inside
+    # the attention launch (what the bench times) and, a step later, one with the two calls
+    sample = [int(np.argmax(ctx_lens)), int(np.argmin(ctx_lens))] + swapped[:2] + swapped[-2:]
+    sample += [int(b) for b in rng.permutation(B) if int(b) not in sample][: 16 - len(sample)]
+    assert ctx_lens.max() == 32768
+    for layer, fused in ((4, True), (9, False)):
+        before, old = _checksum(pool.pages[layer]), _old_rows_sum(wl, layer)
+        ctx, outs, (n_items, _) = _decode_step(wl, wrapper, [layer], fused=fused)
+        assert n_items > B
+        _check_append(wl, ctx, layer, before, old)
+        want = _oracle_rows(wl, ctx, layer, sample)
+        got = outs[layer].float().cpu().numpy()
+        assert np.isfinite(got).all()
+        err = max_rel_err_per_request(got[sample], want)
+        _announce("config5 layer", layer, "fused" if fused else "two calls", "worst request error", err)
+        assert err <= 2e-2, (layer, fused)
+        for t in tasks:
+            t.step()

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from kvutil import max_rel_err
+from kvutil import max_rel_err_per_request
 from oracle import kv_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -84,7 +84,7 @@ def test_rotating_microbatches_keep_their_kv(rounds):
             for layer in range(L):
                 want = shadow.expect(t, layer, q[layer, pos: pos + n], k[layer, pos: pos + n],
                                      v[layer, pos: pos + n])
-                assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
+                assert max_rel_err_per_request(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
             pos += n
         for c in proc.microbatches[m].ongoing_paged_kvcaches.values():
             used_swap_pages |= bool(c.isswap[: c.page_table.occupied].any())
@@ -122,7 +122,7 @@ def test_offload_reload_and_cancel_through_the_stage_driver():
             for layer in range(L):
                 want = shadow.expect(t, layer, q[layer, pos: pos + n], k[layer, pos: pos + n],
                                      v[layer, pos: pos + n])
-                assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (t, layer)
+                assert max_rel_err_per_request(got[layer, pos: pos + n], want) <= 2e-2, (t, layer)
             pos += n
 
     idle = lambda m, **kw: proc.run_step(StepRequest(m, None, **kw))
@@ -203,7 +203,7 @@ def test_scheduler_policies_under_page_pressure(policy):
                 for layer in range(L):
                     want = shadow.expect(t, layer, chunk[:, layer, :HQ], chunk[:, layer, HQ:HQ + HKV],
                                          chunk[:, layer, HQ + HKV:])
-                    assert max_rel_err(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
+                    assert max_rel_err_per_request(got[layer, pos: pos + n], want) <= 2e-2, (step, t, layer)
                 pos += n
         # a task that has produced its budget of tokens is cancelled on its next round;
         # one that is still prefilling has no next input yet and drops out of the batch

@@ -1,12 +1,14 @@
 """Parity of the HIP path (through the C ABI) against the CPU oracle on a real
 MI355X.  Copy-type operators must be bit-exact; attention must stay within
-2e-2 of the fp32 oracle, measured as max |got - ref| / max |ref| (error relative
-to the output's scale), for 16-bit storage and 1e-4 for fp32 storage."""
+2e-2 of the fp32 oracle for 16-bit storage and 1e-4 for fp32 storage, measured as
+max |got - ref| / max |ref| over ONE output row (one request in decode, one query
+position in prefill: all its heads and dims) - every row against its own scale, the
+worst row counts."""
 import numpy as np
 import pytest
 import torch
 
-from kvutil import from_torch, make_scenario, max_rel_err, to_torch, torch_dtype
+from kvutil import from_torch, make_scenario, max_rel_err, max_rel_err_per_request, to_torch, torch_dtype
 from oracle import c_oracle
 from oracle import kv_oracle as orc
 
@@ -145,7 +147,7 @@ def test_decode_attention_matches_oracle(case):
                                 sc.kv_last_page_lens, dtype)
     live = np.asarray(lens) > 0
     assert np.isfinite(got).all()
-    assert max_rel_err(got[live], want[live]) <= ATTN_TOL[dtype]
+    assert max_rel_err_per_request(got[live], want[live]) <= ATTN_TOL[dtype]
     assert not got[~live].any()                       # a request without tokens yields zeros
     if name == "split":
         assert n_items > len(lens)
@@ -196,7 +198,7 @@ def test_decode_attention_is_bitwise_repeatable_across_launches():
         first = w.forward(q, pages).clone()
         want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
                                     sc.kv_last_page_lens, "bf16")
-        assert max_rel_err(first.float().cpu().numpy(), want) <= 2e-2
+        assert max_rel_err_per_request(first.float().cpu().numpy(), want) <= 2e-2
         outs = [w.forward(q, pages) for _ in range(200)]
         torch.cuda.synchronize()
         for i, o in enumerate(outs):
@@ -260,7 +262,7 @@ def test_prefill_attention_matches_oracle(case):
         want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
                                      sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
         assert np.isfinite(got).all()
-        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (name, causal)
+        assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (name, causal)
     w.end_forward()
 
 
@@ -295,7 +297,7 @@ def test_prefill_attention_random_shapes():
         want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
                                      sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
         assert np.isfinite(got).all()
-        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, qo, causal)
+        assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, qo, causal)
         done += 1
 
 
@@ -318,7 +320,7 @@ def test_decode_attention_random_shapes():
         want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
                                     sc.kv_last_page_lens, dtype)
         assert np.isfinite(got).all()
-        assert max_rel_err(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, target)
+        assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, target)
         done += 1
 
 
@@ -351,7 +353,7 @@ def test_decode_with_fused_append_equals_append_then_decode(case):
     assert _same_bits(from_torch(out_b, dtype), from_torch(out_a, dtype))
     want = c_oracle.decode_attn(sc.q, want_pages, sc.kv_page_indices, sc.kv_page_indptr,
                                 sc.kv_last_page_lens, dtype)
-    assert max_rel_err(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
+    assert max_rel_err_per_request(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
     with pytest.raises(ValueError):
         w.forward(q, pages_b, k_append=k)
     with pytest.raises(ValueError):
@@ -392,7 +394,7 @@ def test_decode_with_rope_inside_equals_rope_append_then_decode(case):
                         sc.kv_page_indptr, sc.kv_last_page_lens)
     want = c_oracle.decode_attn(to_storage(q_ref, dtype), want_pages, sc.kv_page_indices,
                                 sc.kv_page_indptr, sc.kv_last_page_lens, dtype)
-    assert max_rel_err(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
+    assert max_rel_err_per_request(out_b.float().cpu().numpy(), want) <= ATTN_TOL[dtype]
     w.end_forward()
 
 
@@ -423,7 +425,7 @@ def test_prefill_with_one_query_equals_decode():
     w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                     _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P)
     pre = w.forward(to_torch(sc.q, "bf16"), to_torch(sc.pages, "bf16")).float().cpu().numpy()
-    assert max_rel_err(pre, dec) < 1e-2
+    assert max_rel_err_per_request(pre, dec) < 1e-2
 
 
 # ------------------------------------------------------------------ rope
@@ -493,10 +495,10 @@ def test_baseline_config1_fp32_append_then_decode():
     w.begin_forward(args[2], args[1], args[3], 32, 8, 128, 16)
     got = w.forward(to_torch(sc.q, "f32"), pages).cpu().numpy()
     assert _same_bits(from_torch(pages, "f32"), want_pages)
-    assert max_rel_err(got, want) <= 1e-4
+    assert max_rel_err_per_request(got, want) <= 1e-4
     # the same problem in bf16 storage stays within the 16-bit tolerance of the fp32 answer
     scb = make_scenario(1, kv_lens=[512] * 8, qo_lens=[1] * 8, dtype="bf16", spare_pages=0)
     got_b, _ = _run_decode(scb)
     want_b = orc.decode_attention(scb.q, scb.pages, scb.kv_page_indices, scb.kv_page_indptr,
                                   scb.kv_last_page_lens, "bf16")
-    assert max_rel_err(got_b, want_b) <= 2e-2
+    assert max_rel_err_per_request(got_b, want_b) <= 2e-2
