@@ -37,6 +37,10 @@ _SIGNATURES = {
     "dskv_decode_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
                                    c_int32, c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32,
                                    c_int32, c_float, c_int32, c_void_p]),
+    "dskv_decode_attn_noalloc_max_bytes": (c_int64, []),
+    "dskv_decode_attn_noalloc": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
+                                           c_int32, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                           c_float, c_int32, c_void_p]),
     "dskv_decode_attn_phases": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_int32, c_int32, c_void_p, c_int64, c_int32, c_int32,
                                           c_int32, c_int32, c_int32, c_float, c_int32, c_int32,

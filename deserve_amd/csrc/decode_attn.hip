@@ -37,6 +37,7 @@
 
 #include <algorithm>
 #include <math.h>
+#include <mutex>
 #include <vector>
 
 namespace dskv {
@@ -53,6 +54,9 @@ constexpr int kMaxWorkgroups = 4096;
 #define DSKV_DECODE_MIN_TILES 4
 #endif
 constexpr int kMinTilesPerWorkgroup = DSKV_DECODE_MIN_TILES;
+#ifndef DSKV_DECODE_STATIC_SCRATCH_BYTES
+#define DSKV_DECODE_STATIC_SCRATCH_BYTES (32 << 20)
+#endif
 
 // Work item written by the planner.  slot < 0: the item covers its whole request
 // and writes the final output row; otherwise it writes partial slot `slot`.
@@ -820,6 +824,77 @@ extern "C" int dskv_decode_rope_append_attn(void *out, const void *q, const void
     return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
                             workspace, workspace_bytes, batch, n_qo_heads, n_kv_heads, head_dim,
                             page_size, sm_scale, dtype, phases, stream, k_new, v_new, rope_table);
+}
+
+// ---------------------------------------------------------------------------
+// The entry point that allocates nothing: the partial results live in a
+// file-scope device array instead of a caller workspace.
+// ---------------------------------------------------------------------------
+namespace dskv {
+
+constexpr int64_t kStaticScratchBytes = DSKV_DECODE_STATIC_SCRATCH_BYTES;
+// Partials (O, m, l) of requests cut by share boundaries.  One copy per GPU, held until the
+// process ends.  Never named in a kernel argument or a copy: host code uses the per-device
+// address that hipGetSymbolAddress returns (the name is a host-side stand-in only).
+static __device__ __align__(256) char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];   // per device: where that GPU's copy of `scratch` lies
+static std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`; resolved on the first call per device.
+static int static_scratch(void **ptr_out)
+{
+    int dev = -1;
+    DSKV_HIP(hipGetDevice(&dev));
+    DSKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "decode_attn_noalloc: device %d outside [0, %d)", dev,
+                 kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        DSKV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        DSKV_REQUIRE(p, "decode_attn_noalloc: the scratch array has no device address");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr_out = g_scratch_ptr[dev];
+    return 0;
+}
+
+}  // namespace dskv
+
+extern "C" int64_t dskv_decode_attn_noalloc_max_bytes(void) { return dskv::kStaticScratchBytes; }
+
+extern "C" int dskv_decode_attn_noalloc(void *out, const void *q, const void *pages_layer,
+                                        const int32_t *kv_page_indices, const int32_t *plan_dev,
+                                        int32_t n_items, int32_t n_workgroups, int32_t batch,
+                                        int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                                        int32_t page_size, float sm_scale, int32_t dtype,
+                                        void *stream)
+{
+    using namespace dskv;
+    if (batch <= 0 || n_items <= 0)
+        return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items,
+                                n_workgroups, nullptr, 0, batch, n_qo_heads, n_kv_heads, head_dim,
+                                page_size, sm_scale, dtype, 3, stream, nullptr, nullptr, nullptr);
+    DSKV_REQUIRE(n_qo_heads > 0 && head_dim > 0, "decode_attn_noalloc: bad shape");
+    DSKV_REQUIRE(n_items >= batch, "decode_attn_noalloc: plan has fewer items than requests");
+    // Every cut adds one item, and a request cut c times owns c + 1 partial slots: the plan
+    // uses at most min(n_items, 2 * (n_items - batch)) slots.
+    const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
+    const int64_t slots = std::min<int64_t>(n_items, 2 * ((int64_t)n_items - batch));
+    if (slots * slot_bytes > kStaticScratchBytes) {
+        set_error("decode_attn_noalloc: %lld partial slots of %lld bytes exceed the built-in scratch "
+                  "of %lld bytes; plan fewer workgroups or pass a workspace to dskv_decode_attn",
+                  (long long)slots, (long long)slot_bytes, (long long)kStaticScratchBytes);
+        return DSKV_E_NOMEM;
+    }
+    void *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    // nothing in the array has to start at zero: every slot the merge pass reads has been
+    // written by the attention pass of the same call
+    return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
+                            ws, kStaticScratchBytes, batch, n_qo_heads, n_kv_heads, head_dim,
+                            page_size, sm_scale, dtype, 3, stream, nullptr, nullptr, nullptr);
 }
 
 extern "C" int dskv_decode_attn(void *out, const void *q, const void *pages_layer,

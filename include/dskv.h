@@ -110,6 +110,25 @@ int dskv_decode_attn(void *out, const void *q, const void *pages_layer,
                      int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
                      float sm_scale, int32_t dtype, void *stream);
 /*
+ * dskv_decode_attn for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and result as dskv_decode_attn, bit for bit, minus the
+ * workspace: the partial results of cut requests go to an array built into the library
+ * (dskv_decode_attn_noalloc_max_bytes() bytes, 32 MiB, one copy per GPU for the life of the
+ * process).  Calls no hipMalloc / hipFree.  A plan whose partials do not fit -
+ * min(n_items, 2 * (n_items - batch)) * n_qo_heads * (head_dim + 2) * 4 bytes - is refused
+ * with DSKV_E_NOMEM.  All calls on one GPU share the array: calls that overlap on one GPU
+ * (two streams, two threads) race; calls on one stream do not.  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress); make that call outside a capture.
+ */
+int64_t dskv_decode_attn_noalloc_max_bytes(void);
+int dskv_decode_attn_noalloc(void *out, const void *q, const void *pages_layer,
+                             const int32_t *kv_page_indices, const int32_t *plan_dev,
+                             int32_t n_items, int32_t n_workgroups, int32_t batch,
+                             int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                             int32_t page_size, float sm_scale, int32_t dtype, void *stream);
+
+/*
  * The same, one pass at a time: phases bit 0 = the split-KV attention pass
  * (writes final rows of uncut requests and the partials of cut ones), bit 1 =
  * the merge pass that combines the partials.  dskv_decode_attn is phases = 3.
