@@ -79,6 +79,9 @@ _SIGNATURES = {
                                            c_int32, c_int32, c_int64, c_int64, c_void_p]),
     "dskv_swap_wait": (c_int32, [c_void_p]),
     "dskv_swap_fence": (c_int32, [c_void_p, c_void_p]),
+    "dskv_swap_query": (c_int32, [c_void_p, POINTER(c_int32)]),
+    "dskv_swap_streams": (c_int32, [c_void_p, POINTER(c_void_p), POINTER(c_void_p)]),
+    "dskv_swap_bind_compute_stream": (c_int32, [c_void_p, c_void_p, POINTER(c_int32)]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -115,12 +118,16 @@ def last_error() -> str:
     return msg.decode() if msg else ""
 
 
+E_INVAL, E_NOMEM, E_STATE = -1, -2, -3
+
+
 def check(rc: int, what: str = "dskv") -> None:
-    """0 ok; negative = argument error -> ValueError; positive = HIP error -> RuntimeError."""
+    """0 ok; argument errors (DSKV_E_INVAL, DSKV_E_NOMEM) -> ValueError; a handle used in
+    the wrong state (DSKV_E_STATE) and HIP errors (positive) -> RuntimeError."""
     if rc == 0:
         return
     msg = f"{what}: {last_error()} (code {rc})"
-    if rc < 0:
+    if rc in (E_INVAL, E_NOMEM):
         raise ValueError(msg)
     raise RuntimeError(msg)
 

@@ -18,6 +18,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <deque>
 #include <new>
 #include <vector>
 
@@ -33,11 +34,21 @@ struct dskv_swap {
     hipEvent_t ids_ready = nullptr;    // page ids have landed on the device
     hipEvent_t gathered[2] = {nullptr, nullptr};   // exchange: chunk left the pool
     hipEvent_t fence = nullptr;
-    // page-id arena: pinned host mirror + device copy, bump-allocated, reset on wait
+    // page-id ring: pinned host mirror + device copy.  A call takes the next free stretch;
+    // a stretch is free again once the events recorded behind the call's last use of it
+    // have completed (checked, never waited for).
     int32_t *ids_host = nullptr;
     int32_t *ids_dev = nullptr;
     int64_t ids_capacity = 0;
-    int64_t ids_used = 0;
+    int64_t ids_head = 0;              // where the next stretch starts
+    struct IdStretch {
+        int64_t begin, end;
+        hipEvent_t done[2];            // per direction stream that read it (null = unused)
+    };
+    std::deque<IdStretch> ids_pending; // oldest first
+    std::vector<hipEvent_t> spare_events;
+    bool probed = false;               // streams checked against the caller's compute stream
+    bool independent = false;          // ... and found to run beside it
 };
 
 namespace dskv {
@@ -56,32 +67,104 @@ static int check_geometry(const char *who, int32_t n_pages, int32_t n_layers,
     return 0;
 }
 
+static void recycle(dskv_swap *h, dskv_swap::IdStretch &st)
+{
+    for (hipEvent_t &e : st.done)
+        if (e) {
+            h->spare_events.push_back(e);
+            e = nullptr;
+        }
+}
+
 static int wait_all(dskv_swap *h)
 {
     for (int d = 0; d < 2; d++) DSKV_HIP(hipStreamSynchronize(h->stream[d]));
-    h->ids_used = 0;
+    for (auto &st : h->ids_pending) recycle(h, st);
+    h->ids_pending.clear();
+    h->ids_head = 0;
     return 0;
 }
 
-// Copy the caller's page ids into the arena and start their upload on `s`: a kernel
-// reading the pinned mirror (slots are multiples of four words, as it wants), so the
-// copy engines carry page data only.
+static int take_event(dskv_swap *h, hipEvent_t *out)
+{
+    if (!h->spare_events.empty()) {
+        *out = h->spare_events.back();
+        h->spare_events.pop_back();
+        return 0;
+    }
+    DSKV_HIP(hipEventCreateWithFlags(out, hipEventDisableTiming));
+    return 0;
+}
+
+// Forget the stretches whose readers have finished (a query, never a wait).
+static void retire_ids(dskv_swap *h)
+{
+    while (!h->ids_pending.empty()) {
+        dskv_swap::IdStretch &st = h->ids_pending.front();
+        for (hipEvent_t e : st.done)
+            if (e && hipEventQuery(e) != hipSuccess) {
+                (void)hipGetLastError();   // hipErrorNotReady is not a failure
+                return;
+            }
+        recycle(h, st);
+        h->ids_pending.pop_front();
+    }
+    if (h->ids_pending.empty()) h->ids_head = 0;
+}
+
+// Copy the caller's page ids into the ring and start their upload on `s`: a kernel
+// reading the pinned mirror (stretches are multiples of four words, as it wants), so the
+// copy engines carry page data only.  Never blocks: when the ring has no free stretch
+// of this size (earlier calls still in flight hold it), the call is refused with
+// DSKV_E_STATE and the caller waits (dskv_swap_wait) or retries later.
 static int stage_ids(dskv_swap *h, const int32_t *ids, int32_t n, hipStream_t s, int32_t **dev_out)
 {
-    const int64_t slot = ((int64_t)n + 3) / 4 * 4;
-    DSKV_REQUIRE(slot <= h->ids_capacity, "swap: %d page ids exceed the engine's limit of %lld", n,
+    const int64_t len = ((int64_t)n + 3) / 4 * 4;
+    DSKV_REQUIRE(len <= h->ids_capacity, "swap: %d page ids exceed the engine's limit of %lld", n,
                  (long long)h->ids_capacity);
-    if (h->ids_used + slot > h->ids_capacity) {
-        int rc = wait_all(h);   // arena full: drain, then start over
-        if (rc) return rc;
+    retire_ids(h);
+    // pending stretches occupy [tail, head) of the ring, possibly wrapped
+    int64_t begin = h->ids_head;
+    const int64_t tail = h->ids_pending.empty() ? begin : h->ids_pending.front().begin;
+    const bool wrapped = !h->ids_pending.empty() && tail >= begin;   // free space is [head, tail)
+    bool fits;
+    if (h->ids_pending.empty()) {
+        begin = 0;
+        fits = true;
+    } else if (wrapped) {
+        fits = begin + len <= tail;
+    } else if (begin + len <= h->ids_capacity) {
+        fits = true;
+    } else {
+        begin = 0;                                   // wrap: free space is [0, tail)
+        fits = len <= tail;
     }
-    int32_t *host = h->ids_host + h->ids_used;
-    int32_t *dev = h->ids_dev + h->ids_used;
+    if (!fits) {
+        set_error("swap: the page-id ring (%lld ids) is held by calls still in flight; wait "
+                  "(dskv_swap_wait) or retry once they have finished", (long long)h->ids_capacity);
+        return DSKV_E_STATE;
+    }
+    int32_t *host = h->ids_host + begin;
+    int32_t *dev = h->ids_dev + begin;
     std::copy(ids, ids + n, host);
-    h->ids_used += slot;
     int rc = dskv_upload_words(dev, host, n, s);
     if (rc) return rc;
+    h->ids_pending.push_back(dskv_swap::IdStretch{begin, begin + len, {nullptr, nullptr}});
+    h->ids_head = begin + len;
     *dev_out = dev;
+    return 0;
+}
+
+// Marks the end of the newest stretch's use on direction `dir` (call after the last kernel
+// that reads it has been enqueued there).
+static int release_ids_after(dskv_swap *h, int dir)
+{
+    dskv_swap::IdStretch &st = h->ids_pending.back();
+    if (!st.done[dir]) {
+        int rc = take_event(h, &st.done[dir]);
+        if (rc) return rc;
+    }
+    DSKV_HIP(hipEventRecord(st.done[dir], h->stream[dir]));
     return 0;
 }
 
@@ -122,6 +205,40 @@ static int close_direction(dskv_swap *h, int dir)
 {
     DSKV_HIP(hipEventRecord(h->dir_done[dir], h->stream[dir]));
     h->dir_used[dir] = true;
+    return release_ids_after(h, dir);
+}
+
+// ---- do two streams run side by side?
+//
+// The HIP runtime maps streams onto a small number of hardware queues (four by default)
+// and packets of one queue run in order: a kernel on a stream that shares its queue with
+// a copy stream waits for the copy.  Which streams share is decided when they are
+// created, from how many streams the process already has - not something a caller can
+// see.  So it is measured: a kernel that idles for half a millisecond goes to one
+// stream, an empty kernel to the other; if the empty one finishes first, the two streams
+// run side by side.
+__global__ void idle_kernel(long ticks)
+{
+    const long t0 = wall_clock64();
+    while (wall_clock64() - t0 < ticks) __builtin_amdgcn_s_sleep(64);
+}
+
+__global__ void empty_kernel() {}
+
+static int runs_beside(hipStream_t a, hipStream_t b, hipEvent_t ea, hipEvent_t eb, long ticks,
+                       bool *beside)
+{
+    DSKV_HIP(hipStreamSynchronize(a));
+    DSKV_HIP(hipStreamSynchronize(b));
+    hipLaunchKernelGGL(idle_kernel, dim3(1), dim3(64), 0, a, ticks);
+    DSKV_HIP(hipEventRecord(ea, a));
+    hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, b);
+    DSKV_HIP(hipEventRecord(eb, b));
+    DSKV_HIP(hipEventSynchronize(eb));
+    const hipError_t q = hipEventQuery(ea);       // still idling = b did not wait for a
+    (void)hipGetLastError();
+    *beside = q == hipErrorNotReady;
+    DSKV_HIP(hipEventSynchronize(ea));
     return 0;
 }
 
@@ -207,6 +324,10 @@ extern "C" int dskv_swap_destroy(dskv_swap_t *h)
     if (h->fence) (void)hipEventDestroy(h->fence);
     for (int i = 0; i < 2; i++)
         if (h->gathered[i]) (void)hipEventDestroy(h->gathered[i]);
+    for (auto &st : h->ids_pending)
+        for (hipEvent_t e : st.done)
+            if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : h->spare_events) (void)hipEventDestroy(e);
     if (h->ids_host) (void)hipHostFree(h->ids_host);
     if (h->ids_dev) (void)hipFree(h->ids_dev);
     delete h;
@@ -325,11 +446,100 @@ extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const vo
     return close_direction(h, 1);
 }
 
+extern "C" int dskv_swap_streams(dskv_swap_t *h, void **out_stream, void **in_stream)
+{
+    DSKV_REQUIRE(h && out_stream && in_stream, "swap_streams: null argument");
+    *out_stream = h->stream[0];
+    *in_stream = h->stream[1];
+    return 0;
+}
+
+extern "C" int dskv_swap_bind_compute_stream(dskv_swap_t *h, void *compute_stream,
+                                             int32_t *independent_out)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h, "swap_bind_compute_stream: null handle");
+    int rc = wait_all(h);
+    if (rc) return rc;
+    hipStream_t compute = (hipStream_t)compute_stream;
+    int khz = 0;
+    DSKV_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, h->device));
+    const long ticks = (long)(khz > 0 ? khz : 100000) / 2;        // half a millisecond
+    hipEvent_t ea = nullptr, eb = nullptr;
+    DSKV_HIP(hipEventCreateWithFlags(&ea, hipEventDisableTiming));
+    DSKV_HIP(hipEventCreateWithFlags(&eb, hipEventDisableTiming));
+    // A stream is good if the compute stream runs beside it, and the second one also runs
+    // beside the first (the two directions of an exchange overlap).  Rejected streams
+    // stay alive until the search is over: the runtime gives a new stream the least
+    // loaded queue, so they steer the next attempt to another queue.
+    std::vector<hipStream_t> rejected;
+    auto good = [&](hipStream_t s, int dir, bool *ok) -> int {
+        bool beside = false;
+        int r = runs_beside(s, compute, ea, eb, ticks, &beside);
+        if (r) return r;
+        if (beside && dir == 1) {
+            r = runs_beside(h->stream[0], s, ea, eb, ticks, &beside);
+            if (r) return r;
+        }
+        *ok = beside;
+        return 0;
+    };
+    bool all_good = true;
+    for (int dir = 0; dir < 2 && rc == 0; dir++) {
+        bool ok = false;
+        rc = good(h->stream[dir], dir, &ok);
+        for (int attempt = 0; rc == 0 && !ok && attempt < 8; attempt++) {
+            hipStream_t fresh = nullptr;
+            hipError_t e = hipStreamCreateWithFlags(&fresh, hipStreamNonBlocking);
+            if (e != hipSuccess) {
+                set_error("swap_bind_compute_stream: hipStreamCreateWithFlags failed: %s",
+                          hipGetErrorString(e));
+                rc = (int)e;
+                break;
+            }
+            rc = good(fresh, dir, &ok);
+            if (rc == 0 && ok) {
+                rejected.push_back(h->stream[dir]);
+                h->stream[dir] = fresh;
+            } else
+                rejected.push_back(fresh);
+        }
+        all_good = all_good && ok;
+    }
+    for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
+    (void)hipEventDestroy(ea);
+    (void)hipEventDestroy(eb);
+    if (rc) return rc;
+    h->probed = true;
+    h->independent = all_good;
+    h->dir_used[0] = h->dir_used[1] = false;      // everything was drained above
+    if (independent_out) *independent_out = all_good ? 1 : 0;
+    return 0;
+}
+
 extern "C" int dskv_swap_wait(dskv_swap_t *h)
 {
     using namespace dskv;
     DSKV_REQUIRE(h, "swap_wait: null handle");
     return wait_all(h);
+}
+
+extern "C" int dskv_swap_query(dskv_swap_t *h, int32_t *done_out)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(h && done_out, "swap_query: null argument");
+    *done_out = 1;
+    for (int d = 0; d < 2; d++) {
+        const hipError_t e = hipStreamQuery(h->stream[d]);
+        if (e == hipErrorNotReady) {
+            (void)hipGetLastError();
+            *done_out = 0;
+        } else if (e != hipSuccess) {
+            set_error("swap_query: hipStreamQuery failed: %s", hipGetErrorString(e));
+            return (int)e;
+        }
+    }
+    return 0;
 }
 
 extern "C" int dskv_swap_fence(dskv_swap_t *h, void *stream)

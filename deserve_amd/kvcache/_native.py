@@ -48,14 +48,44 @@ def scatter_pages(pool, ids: torch.Tensor, chunk: torch.Tensor) -> None:
 
 
 class SwapEngine:
-    """Owner of one dskv_swap handle (side streams + staging buffers)."""
+    """Owner of one dskv_swap handle (two side streams + staging buffers).
 
-    def __init__(self, staging_bytes: int = 128 << 20) -> None:
+    The engine's streams must not share a hardware queue with the stream that computes, or
+    nothing overlaps; which streams share is an accident of how many streams the process
+    has created.  So the engine checks its streams against the current torch stream when
+    it is created (``bind``; half a millisecond per check) and replaces one that
+    serialises.  ``independent`` tells whether a pair that runs beside compute was found."""
+
+    def __init__(self, staging_bytes: int = 128 << 20, bind: bool = True) -> None:
         import ctypes
 
         h = ctypes.c_void_p()
         _lib.check(_lib.lib().dskv_swap_create(ctypes.byref(h), staging_bytes), "swap_create")
         self._h = h
+        self.staging_bytes = staging_bytes
+        self.independent: Optional[bool] = None
+        if bind:
+            self.bind()
+
+    def bind(self, compute_stream: Optional[int] = None) -> bool:
+        """Blocking set-up: make the engine's streams run beside ``compute_stream`` (raw
+        handle; default: the current torch stream) and beside each other."""
+        import ctypes
+
+        ok = ctypes.c_int32(0)
+        stream = _lib.current_stream() if compute_stream is None else compute_stream
+        _lib.check(_lib.lib().dskv_swap_bind_compute_stream(self._h, stream, ctypes.byref(ok)),
+                   "swap_bind_compute_stream")
+        self.independent = bool(ok.value)
+        return self.independent
+
+    def streams(self) -> tuple:
+        """Raw handles (out, in) of the engine's two streams."""
+        import ctypes
+
+        a, b = ctypes.c_void_p(), ctypes.c_void_p()
+        _lib.check(_lib.lib().dskv_swap_streams(self._h, ctypes.byref(a), ctypes.byref(b)), "swap_streams")
+        return a.value, b.value
 
     def close(self) -> None:
         if self._h:
@@ -99,6 +129,14 @@ class SwapEngine:
 
     def wait(self) -> None:
         _lib.check(_lib.lib().dskv_swap_wait(self._h), "swap_wait")
+
+    def done(self) -> bool:
+        """Whether everything enqueued so far has finished (does not block)."""
+        import ctypes
+
+        flag = ctypes.c_int32(0)
+        _lib.check(_lib.lib().dskv_swap_query(self._h, ctypes.byref(flag)), "swap_query")
+        return bool(flag.value)
 
     def fence(self) -> None:
         """Make the current torch stream wait for everything enqueued so far."""

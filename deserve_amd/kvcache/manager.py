@@ -27,7 +27,11 @@ class KVCacheManager:
         self.virtual_page_pool = virtual_page_pool
         self.cpu_chunk_pool = cpu_chunk_pool
         self.page_table_allocator = page_table_allocator
-        self.engine = _native.SwapEngine(staging_bytes)
+        # the pool's engine (its two streams also carry the bulk slice swap) unless another
+        # staging size is asked for
+        shared = getattr(virtual_page_pool, "engine", None)
+        self.engine = shared if shared is not None and staging_bytes == shared.staging_bytes \
+            else _native.SwapEngine(staging_bytes)
 
     def copy_gpu_to_cpu(self, paged_kvcache: PagedKVCache[VirtualPagePool],
                         task_id: str) -> ChunkHandle:

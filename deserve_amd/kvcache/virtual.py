@@ -37,7 +37,7 @@ class CopiedPinnedMemory(PinnedMemory):
 class VirtualPagePool(GpuPagePool):
     def __init__(self, num_layers: int, num_pages_main: int, num_pages_swap: int, page_size: int,
                  main_device: torch.device, main_dtype: torch.dtype, n_kv_heads: int = 8,
-                 head_dim: int = 128):
+                 head_dim: int = 128, swap_staging_bytes: int = 128 << 20):
         super().__init__(num_layers, num_pages_main + 2 * num_pages_swap, page_size, main_device,
                          main_dtype, n_kv_heads, head_dim)
         m, s = num_pages_main, num_pages_swap
@@ -48,9 +48,18 @@ class VirtualPagePool(GpuPagePool):
         self.swap_bitmap = torch.ones((s,), dtype=torch.bool)
         self.swap_count = s
         self.on = 0
-        on_gpu = self.main_device.type == "cuda"
-        self.stream = torch.cuda.Stream(device=self.main_device) if on_gpu else None
-        self.stream2 = torch.cuda.Stream(device=self.main_device) if on_gpu else None
+        # The two side streams of the reference (virtual.py:48-49) are those of one swap
+        # engine, which the per-request offload / reload (KVCacheManager) shares: a stage
+        # process then holds three streams - compute and these two - each on a hardware
+        # queue of its own, which the engine verifies when it is created.
+        self.engine = None
+        self.stream = self.stream2 = None
+        if self.main_device.type == "cuda":
+            with torch.cuda.device(self.main_device):
+                self.engine = _native.SwapEngine(swap_staging_bytes)
+                out_stream, in_stream = self.engine.streams()
+            self.stream = torch.cuda.ExternalStream(out_stream, device=self.main_device)
+            self.stream2 = torch.cuda.ExternalStream(in_stream, device=self.main_device)
 
     def switch(self) -> None:
         """Flip the active slice (virtual.py:54-77): unused prefetched ids go

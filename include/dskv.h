@@ -254,9 +254,12 @@ int dskv_swap_slice(void *slice_base, int64_t layer_stride_bytes, int64_t slice_
  * per-task copies KVCacheManager.copy_gpu_to_cpu / copy_cpu_to_gpu
  * (kvcache/manager.py:24-86); host layout (n_layers*n_pages, page_bytes), layer
  * major then page_ids order.  page_ids is a HOST int32 array (copied at call
- * time); ids outside a layer are refused with DSKV_E_INVAL.  after_stream:
- * work already enqueued there is waited for before the pool is touched.  dskv_swap_wait blocks the host until everything enqueued
- * on the handle is done; dskv_swap_fence makes `stream` wait for it instead.
+ * time, into a ring of 2^20 ids that in-flight calls hold until they have run: a call that
+ * finds the ring full is refused with DSKV_E_STATE - nothing in these calls waits); ids
+ * outside a layer are refused with DSKV_E_INVAL.  after_stream: work already enqueued
+ * there is waited for (on the device) before the pool is touched.  dskv_swap_wait blocks
+ * the host until everything enqueued on the handle is done; dskv_swap_fence makes `stream`
+ * wait for it instead.
  */
 typedef struct dskv_swap dskv_swap_t;
 int dskv_swap_create(dskv_swap_t **handle, int64_t staging_bytes);
@@ -280,6 +283,30 @@ int dskv_swap_exchange_async(dskv_swap_t *handle, void *host_dst, const void *ho
                              int64_t layer_stride_bytes, int64_t page_bytes, void *after_stream);
 int dskv_swap_wait(dskv_swap_t *handle);
 int dskv_swap_fence(dskv_swap_t *handle, void *stream);
+/* Non-blocking: *done_out = 1 if everything enqueued on the handle has finished, else 0. */
+int dskv_swap_query(dskv_swap_t *handle, int32_t *done_out);
+/*
+ * The two side streams of the engine (hipStream_t): [out] device-to-host, [in]
+ * host-to-device.  Lets the bulk slice swap (dskv_swap_slice, the two streams of
+ * kvcache/virtual.py:48-49) run on the engine's streams, so that a process holds three
+ * streams - compute and these two - and not five.
+ */
+int dskv_swap_streams(dskv_swap_t *handle, void **out_stream, void **in_stream);
+/*
+ * Set-up call (blocks; drains the engine and both streams): makes sure the engine's two
+ * streams run beside `compute_stream` and beside each other.  The HIP runtime maps
+ * streams onto a few hardware queues whose packets run in order, and which streams
+ * share a queue depends on how many streams the process created before - a swap whose
+ * stream shares the compute stream's queue does not overlap with compute at all.  The
+ * call measures it (an idling kernel on one stream, an empty one on the other) and
+ * replaces a stream that serialises by a fresh one, up to eight times.
+ * independent_out (may be NULL): 1 if both streams now run beside the compute stream
+ * and each other, 0 if no such pair was found (the engine still works, without overlap).
+ * No counterpart in the reference, whose two torch streams (kvcache/virtual.py:48-49)
+ * are subject to the same sharing.
+ */
+int dskv_swap_bind_compute_stream(dskv_swap_t *handle, void *compute_stream,
+                                  int32_t *independent_out);
 
 #ifdef __cplusplus
 }

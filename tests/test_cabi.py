@@ -73,6 +73,12 @@ def test_argument_errors_return_negative_codes_without_a_gpu():
     assert lib.dskv_swap_slice(16, 64, 128, 2, 16, 16, None, None) == -1             # stride < slice
     assert lib.dskv_swap_slice(None, 0, 0, 0, None, None, None, None) == 0
     assert lib.dskv_swap_wait(None) == -1 and lib.dskv_swap_out_async(None, 1, 1, 1, 1, 1, 64, 64, None) == -1
+    assert lib.dskv_swap_query(None, None) == -1 and lib.dskv_swap_streams(None, None, None) == -1
+    assert lib.dskv_swap_bind_compute_stream(None, None, None) == -1
+    with pytest.raises(RuntimeError):
+        _lib.check(-3, "a handle in the wrong state")
+    with pytest.raises(ValueError):
+        _lib.check(-2, "caller buffer too small")
     with pytest.raises(RuntimeError):
         _lib.check(1, "hip")
 

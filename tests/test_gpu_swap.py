@@ -297,7 +297,8 @@ def test_config3_exchange_overlapped_with_decode_is_bit_exact():
     images_in = [host_image(101), host_image(102)]
     images_out = [pinned_empty(shape, torch.bfloat16), pinned_empty(shape, torch.bfloat16)]
     w, _ = get_wrappers(DEV)
-    eng = _native.SwapEngine()
+    eng = _native.SwapEngine(staging_bytes=images_in[0].numel() * 2)     # one chunk per direction
+    assert eng.independent, "no pair of streams that runs beside the compute stream was found"
 
     def decode_step(outs):
         c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, w)
@@ -389,4 +390,40 @@ def test_config3_exchange_overlapped_with_decode_is_bit_exact():
                                 indptr, c.host["kv_last_page_lens"].numpy(), "bf16")
     got = overlapped[-1].float().cpu().numpy()
     assert max_rel_err_per_request(got, want) <= 2e-2
+    eng.close()
+
+
+def test_swap_calls_never_block_on_a_full_id_ring():
+    """The engine keeps the page ids of calls in flight in a ring of 2^20 entries.  With the
+    engine held up behind a (bounded) sleeping kernel, the call that no longer fits is
+    refused with an error instead of waiting inside an enqueue-only call; once the earlier
+    calls have run, the same call goes through, and every byte arrives."""
+    import time
+
+    from deserve_amd.kvcache import _native
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.pinned.pinned_memory import pinned_empty
+
+    _announce("swap id ring")
+    n = 300_000                                                     # ids per call; 3 calls fit the ring
+    pool = GpuPagePool(1, 64, 1, DEV, torch.float16, n_kv_heads=1, head_dim=4)      # 16-byte pages
+    bits = _fill_random(pool.pages, 77)
+    ids = torch.from_numpy(np.random.default_rng(78).integers(0, 64, size=n).astype(np.int32))
+    hosts = [pinned_empty((n, 2, 1, 1, 4), torch.float16) for _ in range(4)]
+    eng = _native.SwapEngine(8 << 20)
+    torch.cuda.synchronize()
+    torch.cuda._sleep(20_000_000)              # 10 ms at the shader clock, 0.2 s at a 100 MHz counter
+    t0 = time.perf_counter()
+    for h in hosts[:3]:
+        eng.swap_out(h, pool, ids)                                  # wait (on the device) for the sleep
+    with pytest.raises(RuntimeError, match="ring"):
+        eng.swap_out(hosts[3], pool, ids)
+    assert time.perf_counter() - t0 < 0.05, "an enqueue-only call waited"
+    assert not eng.done()
+    eng.wait()
+    eng.swap_out(hosts[3], pool, ids)
+    eng.wait()
+    want = bits[0][ids.numpy()]
+    for h in hosts:
+        assert _same_bits(_bits(h), want)
     eng.close()
