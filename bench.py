@@ -125,6 +125,83 @@ def cpu_baseline(wl, meta, sample_requests: int):
                       f"{med * 1e3:.1f} ms each, scalar C + OpenMP"}
 
 
+def cpu_reference_config1(seed: int):
+    """BASELINE.json configs[0] exactly, on the reference's CPU path restated with torch
+    (oracle/torch_cpu_path.py): one layer, fp32, 32 q / 8 kv heads, head_dim 128, page 16, 8
+    sequences of context 512 after the append, block tables = a seeded random permutation of
+    the 256 pool pages, K/V/Q ~ N(0, 1).  One step = index-assign append of 1 token per
+    sequence, pages[layer, table] gather, repeat_kv + softmax(scores.float()) matmuls.  Warm-up,
+    then the median of 30 steps on all host threads; the HIP path (append kernel + decode
+    attention, fp32 pool) runs the same step beside it and is compared with the CPU output."""
+    import numpy as np
+    import torch
+
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper, append_paged_kv_cache
+    from oracle import torch_cpu_path
+
+    L, Hq, Hkv, D, P, B, N = 1, 32, 8, 128, 16, 8, 512
+    g = torch.Generator().manual_seed(seed + 10)
+    pages = torch.randn((L, 256, 2, P, Hkv, D), generator=g)             # CpuPagePool storage, 32 MiB
+    perm = torch.randperm(256, generator=g)
+    tables = [perm[b * 32: (b + 1) * 32].clone() for b in range(B)]
+    q, k, v = (torch.randn((B, h, D), generator=g) for h in (Hq, Hkv, Hkv))
+    kv_lens = [N] * B
+    threads = torch.get_num_threads()
+    for _ in range(5):
+        out_cpu = torch_cpu_path.decode_step(pages, 0, tables, kv_lens, q, k, v)
+    times = []
+    for _ in range(30):
+        t0 = time.perf_counter()
+        out_cpu = torch_cpu_path.decode_step(pages, 0, tables, kv_lens, q, k, v)
+        times.append(time.perf_counter() - t0)
+    cpu_s = sorted(times)[len(times) // 2]
+    tok_bytes = 2 * Hkv * D * 4
+    nbytes = attention_bytes_per_layer(np.array(kv_lens), 256, B, Hq, D, 4, tok_bytes) + \
+        append_bytes_per_layer(B, B, 256, tok_bytes)
+
+    dev = torch.device("cuda")
+    d_pages = pages[0].to(dev)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    qo, kv_indptr, last = i32(list(range(B + 1))), i32([32 * b for b in range(B + 1)]), i32([P] * B)
+    ids = perm.to(torch.int32).to(dev)
+    dq, dk, dv = q.to(dev), k.to(dev), v.to(dev)
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(16 << 20, dtype=torch.uint8, device=dev))
+    w.begin_forward(kv_indptr, ids, last, Hq, Hkv, D, P)
+
+    def hip_step():
+        append_paged_kv_cache(dk, dv, qo, d_pages, ids, kv_indptr, last)
+        return w.forward(dq, d_pages)
+
+    for _ in range(5):
+        out_hip = hip_step()
+    evs = []
+    for _ in range(30):
+        a_, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a_.record()
+        out_hip = hip_step()
+        b_.record()
+        evs.append((a_, b_))
+    torch.cuda.synchronize()
+    w.end_forward()
+    hip_s = sorted(x.elapsed_time(y) for x, y in evs)[len(evs) // 2] * 1e-3
+    got, want = out_hip.cpu().numpy(), out_cpu.numpy()
+    err = max(float(np.abs(got[b] - want[b]).max() / np.abs(want[b]).max()) for b in range(B))
+    same_pages = bool(torch.equal(d_pages.cpu(), pages[0]))
+    return {"value": round(nbytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "kind": "reference-restatement", "config": "configs[0]",
+            "sample": f"BASELINE.json configs[0] exactly: 1 layer fp32, 8 x 512 tokens after the append, 256-page "
+                      f"pool in a seeded permutation; torch CPU ({threads} threads): index-assign append, "
+                      f"pages[layer, table] gather, repeat_kv + softmax(scores.float()) matmuls; median of 30 "
+                      f"steps after 5 warm-up steps, {cpu_s * 1e3:.3f} ms per step",
+            "ms_per_step": round(cpu_s * 1e3, 4), "algorithmic_bytes_per_step": int(nbytes),
+            "hip_same_config": {"us_per_step": round(hip_s * 1e6, 1), "GBps": round(nbytes / hip_s / 1e9, 1),
+                                "speedup_over_cpu": round(cpu_s / hip_s, 1),
+                                "max_rel_err_vs_cpu_per_request": float(f"{err:.2e}"),
+                                "pages_bit_equal": same_pages,
+                                "note": "append kernel + fp32 decode attention + merge, events on the launch "
+                                        "stream; 32 MiB of KV is launch- and latency-bound on 256 CUs"}}
+
+
 def swap_section(seed: int):
     """Baseline configuration 3 (Llama-3-70B stage, 10 layers, GQA 64q/8kv): one microbatch's
     scattered pages go out to pinned host memory while the next one's come in (one
@@ -163,7 +240,7 @@ def swap_section(seed: int):
         w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
                         last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
                         head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
-                        last_page_len_host=c.host["kv_last_page_lens"])
+                        last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"])
         for layer in range(L):
             pages = wl.pool.get_layered_pages(layer)
             w.forward(wl.q[layer], pages, k_append=wl.k[layer], v_append=wl.v[layer])
@@ -285,7 +362,7 @@ def prefill_section(seed: int):
                     num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
                     qo_indptr_host=c.host["indptr"],
                     paged_kv_indptr_host=c.host["kv_page_indptr"],
-                    paged_kv_last_page_len_host=c.host["kv_last_page_lens"])
+                    paged_kv_last_page_len_host=c.host["kv_last_page_lens"], paged_kv_indices_host=c.host["kv_page_indices"])
     flops = 4 * Hq * D * sum(n * int(p) + n * (n + 1) // 2 for p in prior)
 
     def median_us(fn, reps=5):
@@ -394,7 +471,7 @@ def fragmented_section(seed: int):
         w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
                         last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
                         head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
-                        last_page_len_host=c.host["kv_last_page_lens"])
+                        last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"])
         for layer in range(L):
             pages = pool.get_layered_pages(layer)
             new_kv = dict(k_append=k[layer], v_append=v[layer])   # written by the attention launch
@@ -517,7 +594,7 @@ def main() -> int:
                                      last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
                                      num_kv_heads=Hkv, head_dim=D, page_size=P,
                                      indptr_host=c.host["kv_page_indptr"],
-                                     last_page_len_host=c.host["kv_last_page_lens"],
+                                     last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"],
                                      target_workgroups=a.workgroups)
         for layer in range(L):
             q, k, v = wl.q[layer], wl.k[layer], wl.v[layer]
@@ -623,10 +700,12 @@ def main() -> int:
         times_ms = [x for x in all_ms if x <= 1.5 * all_ms[len(all_ms) // 2]]
         avg_ms = sum(times_ms) / len(times_ms)
         achieved = (sum(attn_bytes_layer) / len(attn_bytes_layer)) / (avg_ms * 1e-3) / 1e9
-        traffic = None
+        traffic = traffic_workload = traffic_alg = None
         tfile = os.path.join(ROOT, "profiles", "decode_attn_cfg2_traffic.json")
         if os.path.exists(tfile):
-            traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
+            tj = json.load(open(tfile))
+            traffic = tj.get("hbm_bytes_per_launch")
+            traffic_workload, traffic_alg = tj.get("workload"), tj.get("algorithmic_bytes_per_launch")
         # cross-checks of the bracketed figure: what a bracket costs with nothing inside it, and
         # the same pass over all layers back to back inside ONE bracket (no cache reuse between
         # layers); bracket - empty bracket, the back-to-back time and rocprofv3 agree
@@ -642,7 +721,7 @@ def main() -> int:
                                      last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
                                      num_kv_heads=Hkv, head_dim=D, page_size=P,
                                      indptr_host=c.host["kv_page_indptr"],
-                                     last_page_len_host=c.host["kv_last_page_lens"],
+                                     last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"],
                                      target_workgroups=a.workgroups)
         scratch_out = torch.empty_like(wl.q[0])
         rounds = 3
@@ -661,6 +740,11 @@ def main() -> int:
                            "empty_bracket_us": round(empty_us, 2), "back_to_back_us": round(b2b_us, 2),
                            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                           "traffic_source": None if traffic is None else
+                           "profiles/decode_attn_cfg2_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an "
+                           "earlier profiled run of this command (" + str(traffic_workload) + ", " +
+                           str(traffic_alg) + " algorithmic bytes per launch there); replayed from that file, "
+                           "not measured in this run",
                            "avg_launch_us": round(avg_ms * 1e3, 2), "launches": len(times_ms),
                            "intervals_left_out": len(all_ms) - len(times_ms),
                            "algorithmic_bytes_per_launch": int(sum(attn_bytes_layer) / len(attn_bytes_layer))}
@@ -697,7 +781,10 @@ def main() -> int:
                         "note": "same step replayed as one HIP graph (host: metadata + plan only)"}
     if not a.no_cpu_baseline:
         meta = {n: last_ctx.host[n].numpy() for n in ("kv_page_indices", "kv_page_indptr", "kv_last_page_lens")}
-        out["cpu_baseline"] = cpu_baseline(wl, meta, sample_requests=16)
+        scalar = cpu_baseline(wl, meta, sample_requests=16)
+        out["cpu_baseline"] = cpu_reference_config1(a.seed)
+        # second figure: the scalar C port on a sample of the benched configuration itself
+        out["cpu_baseline"]["scalar_port_on_benched_config"] = scalar
     del wl, last_ctx
     torch.cuda.empty_cache()
     if not a.no_prefill:

@@ -23,6 +23,9 @@ __global__ __launch_bounds__(256) void move_pages_kernel(char *__restrict__ pool
     const int layer = (int)(r / n_pages);
     const int j = (int)(r - (long)layer * n_pages);
     const long page = page_ids[j];
+    // an id outside the layer moves nothing (callers check ids on the host; this keeps a
+    // bad id that slipped through from addressing outside the pool)
+    if (page < 0 || (page + 1) * page_bytes > layer_stride) return;
     char *p = pool + layer * layer_stride + page * page_bytes;
     char *c = chunk + (long)blockIdx.x * page_bytes;
     const long part_begin = (long)blockIdx.y * kPartBytes;

@@ -105,6 +105,7 @@ class BatchDecode(BatchExec):
                                   last_page_len=ctx.kv_last_page_lens,
                                   indptr_host=ctx.host["kv_page_indptr"],
                                   last_page_len_host=ctx.host["kv_last_page_lens"],
+                                  indices_host=ctx.host["kv_page_indices"],
                                   **self._shape_kwargs())
             self.decode_ctx = ctx
 
@@ -130,6 +131,7 @@ class BatchPrefill(BatchExec):
                                   qo_indptr_host=ctx.host["indptr"],
                                   paged_kv_indptr_host=ctx.host["kv_page_indptr"],
                                   paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"],
+                                  paged_kv_indices_host=ctx.host["kv_page_indices"],
                                   **self._shape_kwargs())
             self.prefill_ctx = ctx
 

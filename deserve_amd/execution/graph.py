@@ -51,9 +51,25 @@ class GraphedDecodeStep:
                                    last_page_len=ctx.kv_last_page_lens,
                                    indptr_host=ctx.host["kv_page_indptr"],
                                    last_page_len_host=ctx.host["kv_last_page_lens"],
+                                   indices_host=ctx.host["kv_page_indices"],
                                    target_workgroups=self.target_workgroups, plan_buffers=self.plan,
                                    **self.shape)
         return ctx
+
+    @staticmethod
+    def graph_key(batch: int, n_workgroups: int, n_items: int, tensors: Sequence[torch.Tensor],
+                  persistent_kernel: bool) -> tuple:
+        """What decides which launches a captured step holds.  Always: batch, workgroup
+        count, whether anything is merged and with which of the two merge kernels (the
+        launcher takes the wide one from 32 parts per request on), input shapes.  The
+        attention kernel of the 16-bit head_dim-128 path is launched with one workgroup per
+        planned workgroup and reads its items from the plan, so the item count is not part
+        of its launch; the generic kernel (fp32 pools, other head dims, groups over 16) is
+        launched with one workgroup per item, so there the item count is part of the key -
+        a replay with another count would skip items or run on stale plan words."""
+        key = (batch, n_workgroups, n_items > batch, n_items > 32 * batch,
+               tuple((tuple(t.shape), t.dtype) for t in tensors))
+        return key if persistent_kernel else key + (n_items,)
 
     def run(self, xs, task_datas: Sequence[TaskData], kvcaches: Sequence[PagedKVCache]) -> torch.Tensor:
         """xs: a tensor or a tuple of tensors, as the stage's forward takes them.  Returns the
@@ -61,12 +77,8 @@ class GraphedDecodeStep:
         tensors = list(xs) if isinstance(xs, (tuple, list)) else [xs]
         ctx = self._prepare(task_datas, kvcaches)
         w = self.wrapper
-        # what decides which kernels a step launches: batch, workgroups, whether anything is
-        # merged and with which of the two merge kernels (the launcher takes the wide one
-        # from 32 parts per request on)
-        batch = len(task_datas)
-        key = (batch, w._n_workgroups, w._n_items > batch, w._n_items > 32 * batch,
-               tuple((tuple(t.shape), t.dtype) for t in tensors))
+        key = self.graph_key(len(task_datas), w._n_workgroups, w._n_items, tensors,
+                             w.fused_append_supported(tensors[0].dtype))
         held = self._graphs.get(key)
         if held is None:
             inputs = [t.clone() for t in tensors]

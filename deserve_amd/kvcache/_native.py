@@ -16,6 +16,17 @@ def _device_ids(ids: torch.Tensor, device: torch.device) -> torch.Tensor:
     return ids.to(device=device, dtype=torch.int32, non_blocking=True).contiguous()
 
 
+def check_page_ids(pool, ids: torch.Tensor, what: str) -> None:
+    """The gather / scatter kernels index the pool by these ids: ids outside [0, num_pages)
+    are refused here, on a host copy (read back, which synchronises, if ids live on the GPU)."""
+    if ids.numel() == 0:
+        return
+    host = ids.detach().cpu()
+    lo, hi = int(host.min()), int(host.max())
+    if lo < 0 or hi >= pool.num_pages:
+        raise ValueError(f"{what}: page ids span [{lo}, {hi}], the pool has pages [0, {pool.num_pages})")
+
+
 def gather_pages(pool, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """pages[:, ids] -> (L, n, 2, P, Hkv, D) contiguous, on the pool's device."""
     n = int(ids.shape[0])
@@ -25,6 +36,7 @@ def gather_pages(pool, ids: torch.Tensor, out: Optional[torch.Tensor] = None) ->
                           device=pool.pages.device)
     if n == 0:
         return out
+    check_page_ids(pool, ids, "gather_pages")
     dev_ids = _device_ids(ids, pool.pages.device)
     rc = _lib.lib().dskv_gather_pages(out.data_ptr(), pool.pages.data_ptr(), dev_ids.data_ptr(), n,
                                       L, pool.layer_stride_bytes, pool.page_bytes, 0, L * n,
@@ -39,7 +51,9 @@ def scatter_pages(pool, ids: torch.Tensor, chunk: torch.Tensor) -> None:
     if n == 0:
         return
     L = pool.num_layers
-    assert chunk.is_contiguous() and chunk.numel() >= L * n * (pool.page_bytes // chunk.element_size())
+    if not chunk.is_contiguous() or chunk.numel() < L * n * (pool.page_bytes // chunk.element_size()):
+        raise ValueError(f"scatter_pages: chunk must be contiguous and hold {L} x {n} pages")
+    check_page_ids(pool, ids, "scatter_pages")
     dev_ids = _device_ids(ids, pool.pages.device)
     rc = _lib.lib().dskv_scatter_pages(pool.pages.data_ptr(), chunk.data_ptr(), dev_ids.data_ptr(),
                                        n, L, pool.layer_stride_bytes, pool.page_bytes, 0, L * n,

@@ -95,6 +95,7 @@ class _PagedWrapper:
         self._workspace = workspace_buffer
         self._planned = False
         self._rope_table, self._rope_key = None, None
+        self._max_page_id = -1
 
     def _shape_args(self, num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> None:
         self._hq, self._hkv, self._d, self._p = num_qo_heads, num_kv_heads, head_dim, page_size
@@ -104,6 +105,38 @@ class _PagedWrapper:
         """Host copy of a small index tensor (synchronises only if none was given)."""
         src = host if host is not None else t.cpu()
         return src.to(torch.int32).contiguous()
+
+    def _check_block_tables(self, h_indptr: torch.Tensor, indices: torch.Tensor,
+                            indices_host: Optional[torch.Tensor]) -> None:
+        """The kernels index the pool by block-table entries: refuse, on the host, tables that
+        are shorter than indptr says or hold a negative id, and remember the largest id so
+        that forward() can refuse a pool that does not have that page."""
+        batch = h_indptr.shape[0] - 1
+        used = int(h_indptr[-1]) if batch > 0 else 0
+        if batch > 0 and (int(h_indptr[0]) != 0 or bool((h_indptr[1:] < h_indptr[:-1]).any())):
+            raise ValueError("kv page indptr must start at 0 and not decrease")
+        if indices.numel() < used:
+            raise ValueError(f"kv page indices hold {indices.numel()} entries, indptr[-1] is {used}")
+        ids = self._host(indices, indices_host)[:used]
+        if indices_host is not None and indices_host.numel() < used:
+            raise ValueError(f"indices_host holds {indices_host.numel()} entries, indptr[-1] is {used}")
+        self._max_page_id = -1
+        if used > 0:
+            lo, hi = int(ids.min()), int(ids.max())
+            if lo < 0:
+                raise ValueError(f"negative page id {lo} in the block tables")
+            self._max_page_id = hi
+
+    def _check_pool(self, paged_kv_data: torch.Tensor, dtype: torch.dtype) -> None:
+        want = (2, self._p, self._hkv, self._d)
+        if paged_kv_data.dim() != 5 or tuple(paged_kv_data.shape[1:]) != want:
+            raise ValueError(f"paged_kv_data must be (num_pages, {', '.join(map(str, want))}) as given to "
+                             f"begin_forward, got {tuple(paged_kv_data.shape)}")
+        if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != dtype:
+            raise ValueError("paged_kv_data must be contiguous and of q's dtype")
+        if self._max_page_id >= paged_kv_data.shape[0]:
+            raise ValueError(f"the block tables name page {self._max_page_id}, the pool has "
+                             f"{paged_kv_data.shape[0]} pages")
 
     def end_forward(self) -> None:
         self._planned = False
@@ -117,14 +150,19 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
                       last_page_len: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
                       head_dim: int, page_size: int, *, indptr_host: Optional[torch.Tensor] = None,
                       last_page_len_host: Optional[torch.Tensor] = None,
+                      indices_host: Optional[torch.Tensor] = None,
                       target_workgroups: int = 0, plan_buffers=None, **_ignored) -> None:
-        """plan_buffers: optional staged upload (an object with staging() / upload(words) /
+        """The *_host arguments are host copies of the index tensors: the planner and the
+        checks of the block tables run on the host; without them the device tensors are read
+        back, which synchronises.
+        plan_buffers: optional staged upload (an object with staging() / upload(words) /
         dev, see model.context.flash.StagedUpload) that receives the work list instead of
         fresh tensors, for callers that replay captured launches."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._indptr, self._indices = _i32(indptr), _i32(indices)
         h_indptr = self._host(indptr, indptr_host)
         h_last = self._host(last_page_len, last_page_len_host)
+        self._check_block_tables(h_indptr, indices, indices_host)
         batch = h_indptr.shape[0] - 1
         L = _lib.lib()
         total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
@@ -180,8 +218,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         q = q.contiguous()
         if tuple(q.shape) != (self._batch, self._hq, self._d):
             raise ValueError(f"q must be ({self._batch}, {self._hq}, {self._d}), got {tuple(q.shape)}")
-        if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != q.dtype:
-            raise ValueError("paged_kv_data must be contiguous and of q's dtype")
+        self._check_pool(paged_kv_data, q.dtype)
         if out is None:
             out = torch.empty_like(q)
         scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
@@ -236,22 +273,30 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
                       num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int, *,
                       qo_indptr_host: Optional[torch.Tensor] = None,
                       paged_kv_indptr_host: Optional[torch.Tensor] = None,
-                      paged_kv_last_page_len_host: Optional[torch.Tensor] = None, **_ignored) -> None:
-        """The *_host arguments are host copies of the index tensors (the planner runs on the
-        host; without them it reads the device tensors back, which synchronises)."""
+                      paged_kv_last_page_len_host: Optional[torch.Tensor] = None,
+                      paged_kv_indices_host: Optional[torch.Tensor] = None, **_ignored) -> None:
+        """The *_host arguments are host copies of the index tensors (the planner and the
+        checks of the block tables run on the host; without them the device tensors are read
+        back, which synchronises)."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
         h_qo = self._host(qo_indptr, qo_indptr_host)
         batch = h_qo.shape[0] - 1
         nnz = int(h_qo[-1]) if batch > 0 else 0
+        if batch > 0 and (int(h_qo[0]) != 0 or bool((h_qo[1:] < h_qo[:-1]).any())):
+            raise ValueError("qo_indptr must start at 0 and not decrease")
+        h_kv = self._host(paged_kv_indptr, paged_kv_indptr_host)
+        if h_kv.shape[0] != h_qo.shape[0]:
+            raise ValueError("qo_indptr and paged_kv_indptr disagree about the batch")
+        self._check_block_tables(h_kv, paged_kv_indices, paged_kv_indices_host)
         L = _lib.lib()
         cap = L.dskv_prefill_plan_bound(batch, nnz)
         block = staging.take(max(cap, 2))
         tiles = block.tensor
         n_tiles = ctypes.c_int32()
         # kv lengths order the tiles longest first
-        h_indptr = self._host(paged_kv_indptr, paged_kv_indptr_host).to(torch.int64)
+        h_indptr = h_kv.to(torch.int64)
         h_last = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host).to(torch.int64)
         n_pages = h_indptr[1:] - h_indptr[:-1]
         kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
@@ -269,8 +314,7 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         q = q.contiguous()
         if tuple(q.shape) != (self._nnz, self._hq, self._d):
             raise ValueError(f"q must be ({self._nnz}, {self._hq}, {self._d}), got {tuple(q.shape)}")
-        if not paged_kv_data.is_contiguous() or paged_kv_data.dtype != q.dtype:
-            raise ValueError("paged_kv_data must be contiguous and of q's dtype")
+        self._check_pool(paged_kv_data, q.dtype)
         out = torch.empty_like(q)
         scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
         rc = _lib.lib().dskv_prefill_attn(

@@ -36,7 +36,7 @@ rope_interleaved             model/layer/attention.py:45-72 and
 
 Pinning status.  The reference has no tests, golden vectors or fixtures for
 this path.  Every allocator model is pinned by the hand-derived known answers
-that follow from the reference source (tests/test_oracle_allocators.py);
+that follow from the reference source (tests/test_allocators.py);
 append/gather/scatter/swap are pinned by brute-force scalar loops and library
 routines (``numpy.take``); attention is pinned by closed forms (kv_len 1,
 constant keys, one dominant key, page-permutation invariance) and by

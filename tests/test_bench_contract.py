@@ -37,5 +37,10 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3 and 0.3 < r["frac"] < 1.0
     c = d["cpu_baseline"]
-    assert c["kind"] in ("port", "reference") and c["cores"] >= 1 and c["value"] > 0 and c["sample"]
+    assert c["kind"] == "reference-restatement" and c["config"] == "configs[0]"
+    assert c["cores"] >= 1 and c["value"] > 0 and c["sample"]
+    h = c["hip_same_config"]
+    assert h["pages_bit_equal"] is True and h["max_rel_err_vs_cpu_per_request"] <= 1e-4 and h["us_per_step"] > 0
+    assert c["scalar_port_on_benched_config"]["kind"] == "port"
+    assert r["traffic"] is None or "not measured in this run" in r["traffic_source"]
     assert d["value"] > 100 * c["value"]            # the GPU path is not the CPU path in disguise

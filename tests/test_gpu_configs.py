@@ -43,7 +43,7 @@ def _decode_step(wl, wrapper, layers, fused=False, rope=False):
                           last_page_len=ctx.kv_last_page_lens, num_qo_heads=a.n_heads,
                           num_kv_heads=a.n_kv_heads, head_dim=a.dim // a.n_heads, page_size=a.page_size,
                           indptr_host=ctx.host["kv_page_indptr"],
-                          last_page_len_host=ctx.host["kv_last_page_lens"])
+                          last_page_len_host=ctx.host["kv_last_page_lens"], indices_host=ctx.host["kv_page_indices"])
     outs = {}
     for layer in layers:
         pages = wl.pool.get_layered_pages(layer)
@@ -163,7 +163,7 @@ def test_config2_llama8b_stage_decode_step_full_size():
         wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ids, last_page_len=ctx.kv_last_page_lens,
                               num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
                               indptr_host=ctx.host["kv_page_indptr"],
-                              last_page_len_host=ctx.host["kv_last_page_lens"])
+                              last_page_len_host=ctx.host["kv_last_page_lens"])    # ids are read back
         again = wrapper.forward(wl.q[7], pages)
         wrapper.end_forward()
         assert torch.equal(again.view(torch.int16), outs[7].view(torch.int16))
@@ -255,7 +255,7 @@ def test_config4_chunked_prefill_full_batch_four_layers():
                     num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P,
                     qo_indptr_host=ctx.host["indptr"],
                     paged_kv_indptr_host=ctx.host["kv_page_indptr"],
-                    paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"])
+                    paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"], paged_kv_indices_host=ctx.host["kv_page_indices"])
     before = [_checksum(pool.pages[l]) for l in range(L)]
     indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
     # slots the chunk will overwrite: positions prior_b .. prior_b + n - 1

@@ -302,6 +302,52 @@ def test_graphed_decode_step_matches_eager_steps():
     assert step.captures == 2 and len(step._graphs) == 2       # both batch shapes are held for replay
 
 
+def test_graphed_decode_step_on_the_generic_kernel_follows_the_item_count():
+    """head_dim 64 takes the generic attention kernel, which is launched with one workgroup
+    per work item: a captured launch is only valid for its item count.  Contexts grow by a
+    token per step so that the planner's item count changes between steps (5, then 7, ...);
+    every replay must equal the eager step."""
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.execution.graph import GraphedDecodeStep
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.stage import KVStage, StageArgs
+    from deserve_amd.synthetic import make_decode_workload
+
+    print("[case] graphed decode step, generic kernel", flush=True)
+    Lg, hq, hkv, d = 2, 8, 2, 64
+    lens = np.array([100, 37, 63, 15])
+    fresh = lambda: make_decode_workload("gg", lens, Lg, hq, hkv, d, P, torch.bfloat16, headroom_tokens=64,
+                                         seed=21, fill=True)
+    wl_e, wl_g = fresh(), fresh()
+    stage = KVStage(StageArgs(n_heads=hq, n_kv_heads=hkv, dim=hq * d, page_size=P, n_layers=Lg), use_rope=False)
+    wrapper, _ = get_wrappers(DEV)
+    gwrapper = type(wrapper)(torch.empty(8 << 20, dtype=torch.uint8, device=DEV))
+    shape = dict(num_qo_heads=hq, num_kv_heads=hkv, head_dim=d, page_size=P)
+    step = GraphedDecodeStep(stage, gwrapper, max_batch=4, max_pages=256, device=DEV, target_workgroups=4, **shape)
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    counts = []
+    for it in range(12):
+        xs = tuple(torch.randn((Lg, 4, h, d), device=DEV, generator=gen).to(torch.bfloat16) for h in (hq, hkv, hkv))
+        ctx = FlashDecodeCtx.init_paged_decode_ctx(wl_e.tasks, wl_e.caches, wrapper)
+        wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ctx.kv_page_indices,
+                              last_page_len=ctx.kv_last_page_lens, indptr_host=ctx.host["kv_page_indptr"],
+                              last_page_len_host=ctx.host["kv_last_page_lens"],
+                              indices_host=ctx.host["kv_page_indices"], target_workgroups=4, **shape)
+        assert not wrapper.fused_append_supported(torch.bfloat16)
+        counts.append(wrapper._n_items)
+        want = stage.forward(xs, ctx).clone()
+        wrapper.end_forward()
+        got = step.run(xs, wl_g.tasks, wl_g.caches).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (it, counts)
+        assert torch.equal(wl_e.pool.pages.view(torch.int16), wl_g.pool.pages.view(torch.int16)), it
+        for wl in (wl_e, wl_g):
+            for t in wl.tasks:
+                t.step()
+    assert len(set(counts)) > 1, counts                     # the scenario did change the item count
+    assert step.captures == len(set(counts))                # one capture per item count, replays otherwise
+
+
 @pytest.mark.gpu
 def test_staged_uploads_are_exact_and_blocks_wait_for_their_readers():
     """dskv_upload_words through the staging pool: every length (quads + tail words), and a

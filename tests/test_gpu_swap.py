@@ -305,7 +305,7 @@ def test_config3_exchange_overlapped_with_decode_is_bit_exact():
         w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
                         last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
                         head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
-                        last_page_len_host=c.host["kv_last_page_lens"])
+                        last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"])
         for layer in range(L):
             outs.append(w.forward(wl.q[layer], pool.get_layered_pages(layer), k_append=wl.k[layer],
                                   v_append=wl.v[layer]))

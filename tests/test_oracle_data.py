@@ -237,3 +237,29 @@ def test_rope_is_complex_multiplication_by_unit_phasors():
     assert np.allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(x, axis=-1), rtol=1e-5)  # rotation
     zero = orc.rope_interleaved(x, np.array([0, 5], np.int32), np.array([0], np.int32))
     assert np.allclose(zero[0], x[0], atol=1e-7)                               # position 0: identity
+
+
+def test_torch_cpu_path_matches_the_numpy_oracle_on_config1_shape():
+    """oracle/torch_cpu_path.py (the reference's host path restated with torch: index-assign
+    append, pages[layer, table] gather, repeat_kv + softmax(scores.float()) matmuls) against
+    the numpy oracle: same pages after the append bit for bit, same attention within fp32
+    rounding.  A wrong GQA map, slot or gather order fails here."""
+    import torch
+
+    from oracle import torch_cpu_path
+
+    sc = make_scenario(1, kv_lens=[512, 33, 16, 1, 100], qo_lens=[1] * 5, dtype="f32", spare_pages=3)
+    want_pages = sc.pages.copy()
+    orc.append_paged_kv(want_pages, sc.k, sc.v, sc.qo_indptr, sc.kv_page_indices, sc.kv_page_indptr,
+                        sc.kv_last_page_lens)
+    want = orc.decode_attention(sc.q, want_pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                sc.kv_last_page_lens, "f32")
+    pages = torch.from_numpy(np.stack([np.zeros_like(sc.pages), sc.pages.copy()]))      # layer 1 of 2
+    tables = [torch.from_numpy(sc.kv_page_indices[sc.kv_page_indptr[b]: sc.kv_page_indptr[b + 1]].astype(np.int64))
+              for b in range(5)]
+    got = torch_cpu_path.decode_step(pages, 1, tables, [int(n) for n in sc.kv_lens], torch.from_numpy(sc.q),
+                                     torch.from_numpy(sc.k), torch.from_numpy(sc.v))
+    assert np.array_equal(pages[1].numpy(), want_pages) and not pages[0].any()
+    assert got.shape == (5, sc.Hq, sc.D)
+    for b in range(5):
+        assert np.abs(got[b].numpy() - want[b]).max() <= 1e-5 * np.abs(want[b]).max(), b
