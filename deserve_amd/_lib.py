@@ -23,9 +23,9 @@ _lib: Optional[ctypes.CDLL] = None
 _SIGNATURES = {
     "dskv_last_error": (c_char_p, []),
     "dskv_version": (c_int32, []),
-    "dskv_append_paged_kv": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                       c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
-                                       c_int32, c_void_p]),
+    "dskv_append_paged_kv": (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
+                                       c_int32, c_int32, c_void_p]),
     "dskv_gather_pages": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int64,
                                     c_int64, c_int64, c_int64, c_void_p]),
     "dskv_scatter_pages": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int64,
@@ -64,8 +64,8 @@ _SIGNATURES = {
     "dskv_apply_rope": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
                                   c_void_p]),
-    "dskv_rope_append_paged_kv": (c_int32, [c_void_p] * 10 + [c_int32] * 6 + [c_float, c_int32,
-                                                                        c_void_p]),
+    "dskv_rope_append_paged_kv": (c_int32, [c_void_p, c_void_p, c_int32] + [c_void_p] * 8 +
+                                  [c_int32] * 6 + [c_float, c_int32, c_void_p]),
     "dskv_upload_words": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "dskv_swap_slice": (c_int32, [c_void_p, c_int64, c_int64, c_int32, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),

@@ -15,6 +15,7 @@ struct AppendTarget {
     const char *v;               // (nnz, Hkv, D) values to store next to K
     const int32_t *kv_indices, *kv_indptr, *kv_last;
     int page_size;
+    int num_pages;               // pages in the layer: an id outside [0, num_pages) is never written
 };
 
 template <int DT>
@@ -46,6 +47,7 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
         const long p = kv_len - (qo_indptr[lo + 1] - qo_indptr[lo]) + (t - qo_indptr[lo]);
         if (n_pages <= 0 || p < 0 || p >= kv_len) return;   // malformed metadata: touch nothing
         const long page = tgt.kv_indices[page_begin + (int)(p / tgt.page_size)];
+        if (page < 0 || page >= tgt.num_pages) return;      // an id outside the pool: touch nothing
         const long half = (long)tgt.page_size * kv_row_bytes;
         k_dst = tgt.pages + page * 2 * half + (p % tgt.page_size) * kv_row_bytes;
         v_dst = k_dst + half;
@@ -155,12 +157,13 @@ extern "C" int dskv_apply_rope(void *q_out, void *k_out, const void *q, const vo
                                int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
                                int32_t head_dim, float rope_theta, int32_t dtype, void *stream)
 {
-    dskv::AppendTarget none = {nullptr, nullptr, nullptr, nullptr, nullptr, 1};
+    dskv::AppendTarget none = {nullptr, nullptr, nullptr, nullptr, nullptr, 1, 0};
     return dskv::launch_rope(q_out, k_out, q, k, qo_indptr, offsets, batch, nnz, n_qo_heads,
                              n_kv_heads, head_dim, rope_theta, dtype, none, stream, "apply_rope");
 }
 
-extern "C" int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, const void *q,
+extern "C" int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, int32_t num_pages,
+                                         const void *q,
                                          const void *k, const void *v, const int32_t *qo_indptr,
                                          const int32_t *offsets, const int32_t *kv_page_indices,
                                          const int32_t *kv_page_indptr,
@@ -174,9 +177,10 @@ extern "C" int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, const v
         DSKV_REQUIRE(pages_layer && v && kv_page_indices && kv_page_indptr && kv_last_page_len,
                      "rope_append: null pointer argument");
         DSKV_REQUIRE(page_size > 0, "rope_append: page_size must be positive");
+        DSKV_REQUIRE(num_pages > 0, "rope_append: num_pages must be positive, got %d", num_pages);
     }
     AppendTarget tgt = {(char *)pages_layer, (const char *)v, kv_page_indices, kv_page_indptr,
-                        kv_last_page_len, page_size};
+                        kv_last_page_len, page_size, num_pages};
     return launch_rope(q_out, nullptr, q, k, qo_indptr, offsets, batch, nnz, n_qo_heads, n_kv_heads,
                        head_dim, rope_theta, dtype, tgt, stream, "rope_append");
 }

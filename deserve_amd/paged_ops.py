@@ -38,7 +38,7 @@ def append_paged_kv_cache(append_key: torch.Tensor, append_value: torch.Tensor,
             or v.dtype != paged_kv_data.dtype:
         raise ValueError("append_key/append_value must be (nnz, Hkv, D) of the pool's dtype")
     rc = _lib.lib().dskv_append_paged_kv(
-        paged_kv_data.data_ptr(), k.data_ptr(), v.data_ptr(), _i32(append_indptr).data_ptr(),
+        paged_kv_data.data_ptr(), paged_kv_data.shape[0], k.data_ptr(), v.data_ptr(), _i32(append_indptr).data_ptr(),
         _i32(kv_indices).data_ptr(), _i32(kv_indptr).data_ptr(), _i32(kv_last_page_len).data_ptr(),
         append_indptr.shape[0] - 1, k.shape[0], P, Hkv, D, k.element_size(), _lib.current_stream())
     _lib.check(rc, "append_paged_kv_cache")
@@ -79,7 +79,7 @@ def rope_append_paged_kv_cache(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
         raise ValueError("q/k/v must be (nnz, H, D) of the pool's dtype")
     q_out = torch.empty_like(q)
     rc = _lib.lib().dskv_rope_append_paged_kv(
-        q_out.data_ptr(), paged_kv_data.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        q_out.data_ptr(), paged_kv_data.data_ptr(), paged_kv_data.shape[0], q.data_ptr(), k.data_ptr(), v.data_ptr(),
         _i32(indptr).data_ptr(), _i32(offsets).data_ptr(), _i32(kv_indices).data_ptr(),
         _i32(kv_indptr).data_ptr(), _i32(kv_last_page_len).data_ptr(), indptr.shape[0] - 1,
         q.shape[0], P, q.shape[1], Hkv, D, float(rope_theta), _lib.dtype_code(q.dtype),

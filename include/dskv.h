@@ -38,9 +38,11 @@ int dskv_version(void);
  * pages_layer: (num_pages, 2, page_size, n_kv_heads, head_dim) of one layer.
  * k, v: (nnz, n_kv_heads, head_dim) contiguous.  All int32 arrays on device.
  * Token i of request b goes to position kv_len_b - n_b + i of that request.
- * Pure byte copy: elt_bytes is 2 or 4.
+ * Pure byte copy: elt_bytes is 2 or 4.  A token whose metadata is inconsistent or
+ * whose page id lies outside [0, num_pages) is skipped: nothing outside the layer
+ * is ever written.
  */
-int dskv_append_paged_kv(void *pages_layer, const void *k, const void *v,
+int dskv_append_paged_kv(void *pages_layer, int32_t num_pages, const void *k, const void *v,
                          const int32_t *qo_indptr, const int32_t *kv_page_indices,
                          const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
                          int32_t batch, int32_t nnz, int32_t page_size, int32_t n_kv_heads,
@@ -228,8 +230,8 @@ int dskv_apply_rope(void *q_out, void *k_out, const void *q, const void *k,
  * never makes a round trip through a temporary.  Bit-identical to
  * dskv_apply_rope followed by dskv_append_paged_kv.
  */
-int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, const void *q, const void *k,
-                              const void *v, const int32_t *qo_indptr, const int32_t *offsets,
+int dskv_rope_append_paged_kv(void *q_out, void *pages_layer, int32_t num_pages, const void *q,
+                              const void *k, const void *v, const int32_t *qo_indptr, const int32_t *offsets,
                               const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
                               const int32_t *kv_last_page_len, int32_t batch, int32_t nnz,
                               int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,

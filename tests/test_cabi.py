@@ -31,12 +31,14 @@ def test_library_exports_every_declared_symbol_and_binding_matches_header():
 
 def test_argument_errors_return_negative_codes_without_a_gpu():
     lib = _lib.lib()
-    assert lib.dskv_append_paged_kv(1, 1, 1, 1, 1, 1, 1, 2, 2, 16, 8, 128, 3, None) == -1
+    assert lib.dskv_append_paged_kv(1, 0, 1, 1, 1, 1, 1, 1, 2, 2, 16, 8, 128, 2, None) == -1
+    assert "num_pages" in _lib.last_error()
+    assert lib.dskv_append_paged_kv(1, 4, 1, 1, 1, 1, 1, 1, 2, 2, 16, 8, 128, 3, None) == -1
     assert "elt_bytes" in _lib.last_error()
     with pytest.raises(ValueError, match="elt_bytes"):
         _lib.check(-1, "append")
-    assert lib.dskv_append_paged_kv(None, None, None, None, None, None, None, 0, 0, 16, 8, 128, 2, None) == 0
-    assert lib.dskv_append_paged_kv(None, 1, 1, 1, 1, 1, 1, 1, 1, 16, 8, 128, 2, None) == -1
+    assert lib.dskv_append_paged_kv(None, 0, None, None, None, None, None, None, 0, 0, 16, 8, 128, 2, None) == 0
+    assert lib.dskv_append_paged_kv(None, 4, 1, 1, 1, 1, 1, 1, 1, 1, 16, 8, 128, 2, None) == -1
     assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 100, 0, 8, None) == -1      # page_bytes % 16
     assert lib.dskv_gather_pages(16, 16, 16, 4, 2, 1024, 64, 3, 9, None) == -1       # row range
     assert lib.dskv_scatter_pages(16, 16, 16, 4, 2, 1024, 64, 0, 0, None) == 0       # empty range

@@ -39,6 +39,11 @@ def test_append_bit_exact(dtype, P):
     cases = {
         "decode": dict(kv_lens=[512, 1, 17, 16, 4096, 33, 250, 15], qo_lens=[1] * 8),
         "chunk": dict(kv_lens=[517, 40, 512, 3, 1029], qo_lens=[512, 40, 7, 3, 0]),
+        # 63 requests is the most whose owner lookup is one vector load; 64 and more take the search
+        "batch63": dict(kv_lens=[20 + 3 * i for i in range(63)], qo_lens=[(i * 7) % 11 for i in range(63)]),
+        "batch64": dict(kv_lens=[20 + 3 * i for i in range(64)], qo_lens=[(i * 5) % 9 for i in range(64)]),
+        "batch200_decode": dict(kv_lens=[1 + (i * 37) % 90 for i in range(200)], qo_lens=[1] * 200),
+        "leading_empty": dict(kv_lens=[10, 10, 40], qo_lens=[0, 0, 25]),
     }
     for name, c in cases.items():
         _announce("append", dtype, P, name)
