@@ -53,6 +53,16 @@ static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole grou
 // than this (log2 domain): probabilities stay below 2^8, the accumulators are
 // rescaled a handful of times per query instead of once per block.
 constexpr float kRescaleSlack = 8.f;
+#ifndef DSKV_PREFILL_LOOKUP_FIRST
+#define DSKV_PREFILL_LOOKUP_FIRST 1
+#endif
+#ifndef DSKV_PREFILL_KREADS_FIRST
+#define DSKV_PREFILL_KREADS_FIRST 0
+#endif
+#ifndef DSKV_PREFILL_SUM_ON_MFMA
+#define DSKV_PREFILL_SUM_ON_MFMA 0
+#endif
+constexpr bool kSumOnMfma = DSKV_PREFILL_SUM_ON_MFMA;   // row sums of P by the matrix pipeline
 
 // Lane roles of the 32x32x16 MFMA, with h = lane / 32 and r = lane % 32:
 //   A operand: row r, k = 8h .. 8h+7.   B operand: column r, k = 8h .. 8h+7.
@@ -131,19 +141,30 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const int n_blocks = (t_end + kBlock - 1) / kBlock;
     // Start value of the running maximum: far below any scaled score, far above a
     // scaled masked score (kNegBig * scale_log2).
-    float m_run[kColTiles], l_run[kColTiles];
+    float m_run[kColTiles];
     f32x16 acc[kColTiles][4];     // O^T: dims 32*dt + 8i + 4h + j of column r in acc[ct][dt][4i + j]
+    // Row sums of P, optionally on the matrix pipeline: ones(32 x tokens) . P^T - every
+    // register of a lane then holds the sum of its column r over the tokens multiplied so
+    // far.  It takes 16 additions per block off the vector pipeline and adds two MFMAs;
+    // measured on MI355X the kernel takes the same time either way, so the default keeps the
+    // sums on the vector pipeline (fewer registers, less matrix work).
+    f32x16 l_acc[kColTiles];
+    float l_run[kColTiles];       // the same sums kept by the vector pipeline (kSumOnMfma off)
     u32x4 pb[kColTiles][2];       // packed probabilities of the previous block, per k-step
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
         m_run[ct] = 0.5f * kNegBig * scale_log2;
         l_run[ct] = 0.f;
 #pragma unroll
+        for (int v = 0; v < 16; v++) l_acc[ct][v] = 0.f;
+#pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[ct][dt][v] = 0.f;
         pb[ct][0] = pb[ct][1] = u32x4{0, 0, 0, 0};
     }
+    const uint32_t one2 = E::pack2(1.f, 1.f);
+    const u32x4 ones = {one2, one2, one2, one2};
 
     // No kv token visible to any row of the tile: the output rows are zero.
     // (Uniform over the workgroup, and before the first barrier.)
@@ -231,51 +252,55 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     // x[4i + j].  Registers 8s .. 8s+7, packed, are the B operand of the P.V MFMA
     // for k-step s, which thereby fixes the tokens of that step's k slots:
     // 16s + 4h + j in slots j, 16s + 8 + 4h + j in slots 4 + j.
-    float x[kColTiles][16];
+    // Two score buffers that the iterations use in turn (S(m) is still being turned into
+    // P(m) while S(m+1) is computed): the loop is unrolled with static phases, so which
+    // buffer is which is known at compile time and no copy is needed.
+    f32x16 xs[2][kColTiles];
     u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
     auto read_k_operands = [&](const char *kst) {
         const char *k_rows = kst + r * kKPitch + h * 16;
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 32);
     };
-    auto scores = [&]() {
-        f32x16 s[kColTiles];
+    auto scores = [&](int buf) {
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) s[ct][v] = 0.f;
+            for (int v = 0; v < 16; v++) xs[buf][ct][v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ks++)
 #pragma unroll
-            for (int ct = 0; ct < kColTiles; ct++) s[ct] = E::mfma_32x32(ka[ks], qreg[ct][ks], s[ct]);
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) x[ct][v] = s[ct][v];
+            for (int ct = 0; ct < kColTiles; ct++)
+                xs[buf][ct] = E::mfma_32x32(ka[ks], qreg[ct][ks], xs[buf][ct]);
     };
-    // Masks block blk's scores (needed from w_mask_from on).
-    auto mask_scores = [&](int blk) {
+    // Masks block blk's scores (needed from w_mask_from on).  The empty volatile statement
+    // keeps this a branch: the compiler otherwise turns it into selects that every block
+    // pays for (48 vector instructions), and only the blocks on the diagonal need it.
+    auto mask_scores = [&](int blk, int buf) {
         const int t = blk * kBlock;
 #pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++)
+        for (int ct = 0; ct < kColTiles; ct++) {
+            asm volatile("" : "+v"(xs[buf][ct]));   // (re)defined here: the selects cannot leave the branch
 #pragma unroll
             for (int v = 0; v < 16; v++)
-                if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit[ct]) x[ct][v] = kNegBig;
+                if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit[ct]) xs[buf][ct][v] = kNegBig;
+        }
     };
-    // Column maximum of the block in x, and whether the running maximum has to be
+    // Column maximum of the block in xs[buf], and whether the running maximum has to be
     // raised before the block's exponentials.
     float m_blk[kColTiles];
     bool raise = false;
-    auto block_max = [&]() {
+    auto block_max = [&](int buf) {
         raise = false;
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
-            const float *xc = x[ct];
-            // scale_log2 > 0: the maximum can be taken before scaling
-            float m = fmaxf(fmaxf(fmaxf(fmaxf(xc[0], xc[1]), fmaxf(xc[2], xc[3])),
-                                  fmaxf(fmaxf(xc[4], xc[5]), fmaxf(xc[6], xc[7]))),
-                            fmaxf(fmaxf(fmaxf(xc[8], xc[9]), fmaxf(xc[10], xc[11])),
-                                  fmaxf(fmaxf(xc[12], xc[13]), fmaxf(xc[14], xc[15]))));
+            const f32x16 &xc = xs[buf][ct];
+            // scale_log2 > 0: the maximum can be taken before scaling.  A chain of
+            // three-input maxima: 8 instructions for 16 values.
+            float m = fmaxf(fmaxf(xc[0], xc[1]), xc[2]);
+#pragma unroll
+            for (int v = 3; v < 15; v += 2) m = fmaxf(fmaxf(m, xc[v]), xc[v + 1]);
+            m = fmaxf(m, xc[15]);
             float other = m;
             swap_halves32(m, other);
             m_blk[ct] = fmaxf(m, other) * scale_log2;
@@ -333,17 +358,24 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     __syncthreads();
     if (w_end > 0) {
         read_k_operands(k_stage[0]);
-        scores();
-        if (kBlock > w_mask_from) mask_scores(0);
-        block_max();
+        scores(0);
+        if (kBlock > w_mask_from) mask_scores(0, 0);
+        block_max(0);
     }
     const int v_lane_off = (4 * h + (c >> 2)) * kPVPitch + (g & 1) * 32 + (c & 3) * 8;
     auto iteration = [&](int m, int phase, RowSet &rows, RowSet &next) {   // phase = m % 4, a literal at each call
         __syncthreads();
         store_rows(k_stage[phase & 1], kKPitch, rows.k);              // K(m+2)
         store_rows(v_stage[(phase + 2) & 3], kPVPitch, rows.v);       // V(m+2)
+#if DSKV_PREFILL_LOOKUP_FIRST
+        // the page lookup goes out before the row loads: vector loads return in order, so the
+        // wait for this lookup (next iteration) then leaves the row loads behind it in flight
+        lookup_pages(m + 6, rows.pg);
+        load_rows(m + 4, rows.desc, rows.k, rows.v);
+#else
         load_rows(m + 4, rows.desc, rows.k, rows.v);
         lookup_pages(m + 6, rows.pg);
+#endif
         if (!(w_end > 0 && (m - 1) * kBlock < w_end)) {
             prepare_rows(m + 5, next.pg, next.desc);
             return;
@@ -356,7 +388,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
                 const float m_new = fmaxf(m_run[ct], m_blk[ct]);
                 const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
                 m_run[ct] = m_new;
-                l_run[ct] *= alpha;
+                if (kSumOnMfma) l_acc[ct] *= alpha;
+                else l_run[ct] *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < 4; dt++) acc[ct][dt] *= alpha;
 #pragma unroll
@@ -377,19 +410,20 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         // with the masking of S(m+1), where needed, between them.  A masked score
         // is kNegBig and the maximum never drops below its start value, so masked
         // probabilities come out as exp2(-huge) = 0 without a select.
-        float s_cur[kColTiles][16];
+        const int cur = phase & 1, nxt = cur ^ 1;   // xs[cur] = S(m), xs[nxt] receives S(m+1)
         u32x4 pb_prev[kColTiles][2];
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
             pb_prev[ct][0] = pb[ct][0];
             pb_prev[ct][1] = pb[ct][1];
-#pragma unroll
-            for (int v = 0; v < 16; v++) s_cur[ct][v] = x[ct][v];
         }
         // V operand: the transposing read hands each block of 16 lanes four tokens
         // of 16 consecutive dims, lane i of the block supplying the address of dims
         // 4*(i%4) .. +3 of the block's token i/4
         read_k_operands(k_stage[(phase + 1) & 1]);                       // K(m+1)
+#if DSKV_PREFILL_KREADS_FIRST
+        __builtin_amdgcn_sched_barrier(0);   // all eight K operands requested before anything else
+#endif
         const char *v_rows = v_stage[(phase + 3) & 3] + v_lane_off;        // V(m-1)
         u32x4 va[4][2];
 #pragma unroll
@@ -401,16 +435,16 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
                 const u32x2 a_hi = read_transposed(vp + 8 * kPVPitch);
                 va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
             }
-        scores();
+        scores(nxt);
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
             float p[16], p_sum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][v], scale_log2, -m_run[ct]));
-                p_sum += p[v];
+                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(xs[cur][ct][v], scale_log2, -m_run[ct]));
+                if (!kSumOnMfma) p_sum += p[v];
             }
-            l_run[ct] += p_sum;
+            if (!kSumOnMfma) l_run[ct] += p_sum;
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
                 pb[ct][ks] = u32x4{E::pack2(p[8 * ks], p[8 * ks + 1]), E::pack2(p[8 * ks + 2], p[8 * ks + 3]),
@@ -418,7 +452,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             // keeps P(m) in this half (it is only consumed by the next iteration)
             asm volatile("" ::"v"(pb[ct][0]), "v"(pb[ct][1]), "v"(l_run[ct]));
         }
-        if ((m + 2) * kBlock > w_mask_from) mask_scores(m + 1);   // wave-uniform
+        if ((m + 2) * kBlock > w_mask_from) mask_scores(m + 1, nxt);   // wave-uniform
 
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
@@ -427,8 +461,14 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ct++)
                     acc[ct][dt] = E::mfma_32x32(va[dt][ks], pb_prev[ct][ks], acc[ct][dt]);
+        if (kSumOnMfma)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int ct = 0; ct < kColTiles; ct++)
+                    l_acc[ct] = E::mfma_32x32(ones, pb_prev[ct][ks], l_acc[ct]);
         prepare_rows(m + 5, next.pg, next.desc);   // for the loads of the next iteration
-        block_max();
+        block_max(nxt);
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
     };
@@ -441,9 +481,12 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
-        float l_other = l_run[ct];
-        swap_halves32(l_run[ct], l_other);
-        const float l = l_run[ct] + l_other;
+        float l = l_acc[ct][0];   // summed over all tokens by the MFMA (both lane halves)
+        if (!kSumOnMfma) {
+            float l_other = l_run[ct];
+            swap_halves32(l_run[ct], l_other);
+            l = l_run[ct] + l_other;
+        }
         if (!live[ct]) continue;
         const float inv = l > 0.f ? 1.f / l : 0.f;
         uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
