@@ -100,12 +100,19 @@ class BuddyIndex:
         if not self.levels[level]:
             donor = next((lv for lv in range(level + 1, self.height) if self.levels[lv]), None)
             if donor is not None:
-                for lv in range(donor, level, -1):
-                    parent = self.levels[lv].pop()
-                    self.levels[lv - 1] += [2 * parent, 2 * parent + 1]
+                self.split(level, donor)
         if not self.levels[level]:
             raise RuntimeError(f"Failed to allocate chunks for size {size} on level {level}")
         return self.levels[level].pop(0), level
+
+    def split(self, begin: int, end: int) -> None:
+        """One chunk of level ``end`` becomes free chunks down to level ``begin``
+        (chunk_pool.py:51-59): at every level on the way the LAST free id is taken and
+        both halves are appended to the level below.  IndexError if a level on the way
+        has no free chunk, as the reference's ``pop()``."""
+        for lv in range(end, begin, -1):
+            parent = self.levels[lv].pop()
+            self.levels[lv - 1] += [2 * parent, 2 * parent + 1]
 
     def release(self, cid: int, level: int) -> None:
         for lv in range(level, self.height):

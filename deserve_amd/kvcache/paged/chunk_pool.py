@@ -43,6 +43,11 @@ class ChunkPool:
     def available_ids(self) -> list:
         return self._buddy.levels
 
+    def split(self, begin: int, end: int) -> None:
+        """Public as in the reference (chunk_pool.py:51-59); like there, the caller holds
+        the mutex or owns the pool."""
+        self._buddy.split(begin, end)
+
     def alloc(self, size: int) -> ChunkHandle:
         with self.mutex:
             cid, level = self._buddy.alloc(size)   # RuntimeError when exhausted

@@ -159,6 +159,23 @@ def test_buddy_known_answers():
         pool.alloc(4)
 
 
+def test_buddy_split_is_public_and_matches_the_reference_walk():
+    """chunk_pool.py:51-59 by hand for height 4: split(0, 3) pops the root (id 0, level 3),
+    appends [0, 1] to level 2, pops the LAST of those (1) and appends [2, 3] to level 1, pops 3
+    and appends [6, 7] to level 0."""
+    from deserve_amd.kvcache.paged.chunk_pool import CpuChunkPool
+
+    pool = CpuChunkPool(1, 4, 1, torch.float32, n_kv_heads=1, head_dim=1)
+    assert pool.available_ids == [[], [], [], [0]]
+    pool.split(0, 3)
+    assert pool.available_ids == [[6, 7], [2], [0], []]
+    pool.split(0, 1)                                    # the last free id of level 1 again
+    assert pool.available_ids == [[6, 7, 4, 5], [], [0], []]
+    with pytest.raises(IndexError):
+        pool.split(0, 1)                                # nothing free at level 1
+    assert pool.alloc(1).id == 6                        # alloc pops the FIRST id of its level
+
+
 def test_buddy_random_alloc_free_returns_to_single_root_and_ranges_are_disjoint():
     rng = np.random.default_rng(1)
     for trial in range(30):
