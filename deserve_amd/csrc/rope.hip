@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
                                                    const int32_t *__restrict__ qo_indptr,
                                                    const int32_t *__restrict__ offsets, int batch,
                                                    int n_qo_heads, int n_kv_heads, int head_dim,
-                                                   float theta, AppendTarget tgt)
+                                                   float theta, AppendTarget tgt, RopeFreqs freqs)
 {
     typedef Chunk<DT> C;
     constexpr int E = C::kElems;
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
 
     float cs[E / 2], sn[E / 2];
 #pragma unroll
-    for (int j = 0; j < E / 2; j++) rope_angle(pos, col * (E / 2) + j, head_dim, theta, cs[j], sn[j]);
+    for (int j = 0; j < E / 2; j++) rope_angle(pos, col * (E / 2) + j, head_dim, theta, freqs, cs[j], sn[j]);
     const long row_bytes = (long)head_dim * (16 / E);
     const int total_heads = n_qo_heads + n_kv_heads;
     for (int h = head_lane; h < total_heads; h += head_lanes) {
@@ -87,14 +87,15 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
 // table[b][D/2 .. D) = sin of positions[b] * theta^(-2*pair/D).
 __global__ __launch_bounds__(256) void rope_table_kernel(float *__restrict__ table,
                                                          const int32_t *__restrict__ positions,
-                                                         int batch, int head_dim, float theta)
+                                                         int batch, int head_dim, float theta,
+                                                         RopeFreqs freqs)
 {
     const int pairs = head_dim / 2;
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= (long)batch * pairs) return;
     const int b = (int)(i / pairs), pair = (int)(i - (long)b * pairs);
     float cs, sn;
-    rope_angle((float)positions[b], pair, head_dim, theta, cs, sn);
+    rope_angle((float)positions[b], pair, head_dim, theta, freqs, cs, sn);
     table[(long)b * head_dim + pair] = cs;
     table[(long)b * head_dim + pairs + pair] = sn;
 }
@@ -120,10 +121,11 @@ static int launch_rope(void *q_out, void *k_out, const void *q, const void *k,
                   (uintptr_t)tgt.pages | (uintptr_t)tgt.v) % 16 == 0,
                  "%s: tensors must be 16-byte aligned", who);
     hipStream_t s = (hipStream_t)stream;
+    const RopeFreqs freqs = rope_freqs(rope_theta, head_dim);
 #define DSKV_LAUNCH_ROPE(DT)                                                                    \
     hipLaunchKernelGGL((rope_kernel<DT>), dim3((unsigned)nnz), dim3(256), 0, s, (char *)q_out,  \
                        (char *)k_out, (const char *)q, (const char *)k, qo_indptr, offsets,     \
-                       batch, n_qo_heads, n_kv_heads, head_dim, rope_theta, tgt)
+                       batch, n_qo_heads, n_kv_heads, head_dim, rope_theta, tgt, freqs)
     if (dtype == DSKV_F32) DSKV_LAUNCH_ROPE(DSKV_F32);
     else if (dtype == DSKV_F16) DSKV_LAUNCH_ROPE(DSKV_F16);
     else DSKV_LAUNCH_ROPE(DSKV_BF16);
@@ -147,7 +149,8 @@ extern "C" int dskv_rope_table(float *table, const int32_t *positions, int32_t b
     DSKV_REQUIRE((uintptr_t)table % 16 == 0, "rope_table: the table must be 16-byte aligned");
     const long n = (long)batch * (head_dim / 2);
     hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, table, positions, batch, head_dim, rope_theta);
+                       (hipStream_t)stream, table, positions, batch, head_dim, rope_theta,
+                       rope_freqs(rope_theta, head_dim));
     DSKV_LAUNCH_CHECK("rope_table_kernel");
     return 0;
 }

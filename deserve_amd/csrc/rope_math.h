@@ -59,13 +59,39 @@ template <> struct Chunk<DSKV_BF16> {
     }
 };
 
-// cos and sin of pos * theta^(-2*pair/D), evaluated as the reference's table does:
-// 1 / theta^(2*pair/D).
-__device__ __forceinline__ void rope_angle(float pos, int pair, int head_dim, float theta,
-                                           float &cs, float &sn)
+// The frequencies 1 / theta^(2*pair/D) of the reference's table (execution/exec.py:44 of
+// the reference: fp32 power of the fp32 quotient 2*pair/D, fp32 reciprocal), computed once per
+// launch on the host and handed to the kernel by value: the angle pos * inv_freq is then the
+// same fp32 product everywhere, and no lane evaluates a power.  The power is taken correctly
+// rounded to fp32 (evaluated in double): fp32 library powers differ from that, and from each
+// other, in the last bit now and then, and at position 4000 one ulp of a frequency is 2e-4 rad.
+// Head dims over 256 (more pairs than the table holds) evaluate the power on the device.
+constexpr int kRopeTablePairs = 128;
+struct RopeFreqs {
+    float inv[kRopeTablePairs];
+    int pairs;   // entries filled; 0: evaluate on the device
+};
+static inline RopeFreqs rope_freqs(float theta, int head_dim)
 {
-    const float inv_freq = 1.0f / powf(theta, (float)(2 * pair) / (float)head_dim);
-    sincosf(pos * inv_freq, &sn, &cs);
+    RopeFreqs f;
+    f.pairs = head_dim / 2 <= kRopeTablePairs ? head_dim / 2 : 0;
+    for (int j = 0; j < kRopeTablePairs; j++)
+        f.inv[j] = j < f.pairs
+                       ? 1.0f / (float)pow((double)theta, (double)((float)(2 * j) / (float)head_dim))
+                       : 0.f;
+    return f;
+}
+
+// cos and sin of pos * theta^(-2*pair/D).
+__device__ __forceinline__ void rope_angle(float pos, int pair, int head_dim, float theta,
+                                           const RopeFreqs &freqs, float &cs, float &sn)
+{
+    const float inv_freq = freqs.pairs > 0 ? freqs.inv[pair]
+                                           : 1.0f / powf(theta, (float)(2 * pair) / (float)head_dim);
+    // the angle is the rounded fp32 product, as in the reference's table (torch.outer of fp32
+    // values): __fmul_rn keeps the compiler from fusing it into the range reduction of sincosf,
+    // which it would do in one kernel and not in another
+    sincosf(__fmul_rn(pos, inv_freq), &sn, &cs);
 }
 
 // (f[2j], f[2j+1]) rotated by the angle whose cosine and sine are cs[j], sn[j].
@@ -74,9 +100,12 @@ __device__ __forceinline__ void rope_rotate(float *f, const float *cs, const flo
 {
 #pragma unroll
     for (int j = 0; j < kPairs; j++) {
+        // one product rounded, the other fused, spelled out: left to the compiler, which of the
+        // two gets fused differs from kernel to kernel, and the fused decode launch must give
+        // the bits of the stand-alone rotation
         const float re = f[2 * j], im = f[2 * j + 1];
-        f[2 * j] = re * cs[j] - im * sn[j];
-        f[2 * j + 1] = re * sn[j] + im * cs[j];
+        f[2 * j] = __fmaf_rn(re, cs[j], -__fmul_rn(im, sn[j]));
+        f[2 * j + 1] = __fmaf_rn(re, sn[j], __fmul_rn(im, cs[j]));
     }
 }
 

@@ -486,6 +486,17 @@ def prefill_attention(q: np.ndarray, qo_indptr: np.ndarray, pages_layer: np.ndar
 # --------------------------------------------------------------------------
 # Rotary embedding, adjacent-pair ("interleaved") convention
 # --------------------------------------------------------------------------
+def rope_inv_freq(theta: float, D: int) -> np.ndarray:
+    """The reference's frequency table, exec.py:44: ``1.0 / (theta ** (arange(0, D, 2).float() / D))``
+    in fp32.  The power is taken correctly rounded to fp32 here (evaluated in double): library
+    fp32 powers (torch's, numpy's, the C library's) agree with that up to the last bit and not
+    always with each other, and at position 4000 one ulp of a frequency is 2e-4 rad of angle.
+    The reciprocal is the fp32 division."""
+    expo = np.arange(0, D, 2, dtype=np.float32) / np.float32(D)
+    power = (np.float64(np.float32(theta)) ** expo.astype(np.float64)).astype(np.float32)
+    return (np.float32(1.0) / power).astype(np.float32)
+
+
 def rope_interleaved(x: np.ndarray, indptr: np.ndarray, offsets: np.ndarray,
                      theta: float = 500000.0) -> np.ndarray:
     """x: (nnz, H, D) fp32.  Token i of request b sits at position
@@ -494,7 +505,7 @@ def rope_interleaved(x: np.ndarray, indptr: np.ndarray, offsets: np.ndarray,
     x = np.asarray(x, dtype=np.float32)
     nnz, H, D = x.shape
     out = np.empty_like(x)
-    inv = (1.0 / (np.float32(theta) ** (np.arange(0, D, 2, dtype=np.float32) / np.float32(D)))).astype(np.float32)
+    inv = rope_inv_freq(theta, D)
     for b in range(len(indptr) - 1):
         for i in range(int(indptr[b + 1] - indptr[b])):
             t = int(indptr[b]) + i
