@@ -236,11 +236,7 @@ def swap_section(seed: int):
     settle_heap()
 
     def decode_step():
-        c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, w)
-        w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
-                        last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
-                        head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
-                        last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"])
+        FlashDecodeCtx.init_and_plan(wl.tasks, wl.caches, w, Hq, Hkv, D, P)
         for layer in range(L):
             pages = wl.pool.get_layered_pages(layer)
             w.forward(wl.q[layer], pages, k_append=wl.k[layer], v_append=wl.v[layer])
@@ -467,11 +463,7 @@ def fragmented_section(seed: int):
 
     def decode_step(record: bool):
         nonlocal attn_bytes
-        c = FlashDecodeCtx.init_paged_decode_ctx(tasks, caches, w)
-        w.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
-                        last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv,
-                        head_dim=D, page_size=P, indptr_host=c.host["kv_page_indptr"],
-                        last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"])
+        c = FlashDecodeCtx.init_and_plan(tasks, caches, w, Hq, Hkv, D, P)
         for layer in range(L):
             pages = pool.get_layered_pages(layer)
             new_kv = dict(k_append=k[layer], v_append=v[layer])   # written by the attention launch
@@ -587,15 +579,10 @@ def main() -> int:
     fused = not a.no_fused_append
 
     def one_step(timed: bool, rope: bool = a.rope):
-        """prepare (metadata + plan, one upload each) then L x (append + attention: one launch
+        """prepare (metadata + plan in one upload) then L x (append + attention: one launch
         for both, or two with --no-fused-append)."""
-        c = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, decode_wrapper)
-        decode_wrapper.begin_forward(indptr=c.kv_page_indptr, indices=c.kv_page_indices,
-                                     last_page_len=c.kv_last_page_lens, num_qo_heads=Hq,
-                                     num_kv_heads=Hkv, head_dim=D, page_size=P,
-                                     indptr_host=c.host["kv_page_indptr"],
-                                     last_page_len_host=c.host["kv_last_page_lens"], indices_host=c.host["kv_page_indices"],
-                                     target_workgroups=a.workgroups)
+        c = FlashDecodeCtx.init_and_plan(wl.tasks, wl.caches, decode_wrapper, Hq, Hkv, D, P,
+                                         target_workgroups=a.workgroups)
         for layer in range(L):
             q, k, v = wl.q[layer], wl.k[layer], wl.v[layer]
             pages = wl.pool.get_layered_pages(layer)

@@ -100,13 +100,9 @@ class BatchDecode(BatchExec):
     def prepare(self) -> None:
         with torch.inference_mode():
             wrapper, _ = get_wrappers(self.kvcaches[0].pool.main_device)
-            ctx = FlashDecodeCtx.init_paged_decode_ctx(self.task_datas, self.kvcaches, wrapper)
-            wrapper.begin_forward(indptr=ctx.kv_page_indptr, indices=ctx.kv_page_indices,
-                                  last_page_len=ctx.kv_last_page_lens,
-                                  indptr_host=ctx.host["kv_page_indptr"],
-                                  last_page_len_host=ctx.host["kv_last_page_lens"],
-                                  indices_host=ctx.host["kv_page_indices"],
-                                  **self._shape_kwargs())
+            # the context's index arrays and the attention work list go up in one kernel
+            ctx = FlashDecodeCtx.init_and_plan(self.task_datas, self.kvcaches, wrapper,
+                                               **self._shape_kwargs())
             self.decode_ctx = ctx
 
     def step(self, ignore_eos: bool) -> BatchResult:

@@ -107,6 +107,15 @@ class MetadataBuffers(StagedUpload):
         super().__init__(5 * ((max_batch + 1 + 3) // 4 * 4) + (max_pages + 3) // 4 * 4, device)
 
 
+def metadata_layout(meta: Dict[str, np.ndarray]):
+    """(start word of every array, total words): each array starts on a 16-byte boundary."""
+    starts, total = {}, 0
+    for f in _FIELDS:
+        starts[f] = total
+        total += (meta[f].shape[0] + 3) // 4 * 4
+    return starts, total
+
+
 def upload_metadata(meta: Dict[str, np.ndarray], device: torch.device,
                     buffers: "MetadataBuffers | None" = None):
     """One pinned staging block, one upload kernel; returns (device views, host views).
@@ -168,6 +177,35 @@ class FlashDecodeCtx(FlashForwardCtx):
                               wrapper: BatchDecodeWithPagedKVCacheWrapper,
                               buffers: "MetadataBuffers | None" = None) -> "FlashDecodeCtx":
         return cls.init_paged_forward_ctx(task_datas, kvcaches, buffers, decode_wrapper=wrapper)
+
+    @classmethod
+    def init_and_plan(cls, task_datas: List[TaskData], kvcaches: List[PagedKVCache[GpuPagePool]],
+                      wrapper: BatchDecodeWithPagedKVCacheWrapper, num_qo_heads: int, num_kv_heads: int,
+                      head_dim: int, page_size: int, target_workgroups: int = 0) -> "FlashDecodeCtx":
+        """init_paged_decode_ctx + wrapper.begin_forward as ONE upload: the six index arrays
+        and the attention work list share a pinned block and reach the device through one
+        kernel (what BatchDecode.prepare does; the reference makes five host-to-device
+        tensor constructions and FlashInfer its own plan upload, flash.py:46-64,
+        exec.py:184-192)."""
+        pool = kvcaches[0].pool
+        meta = build_host_metadata(task_datas, kvcaches)
+        starts, total = metadata_layout(meta)
+        host = {f: torch.from_numpy(meta[f]) for f in _FIELDS}
+
+        def fill(view: torch.Tensor) -> None:
+            arr = view.numpy()
+            for f in _FIELDS:
+                arr[starts[f]: starts[f] + meta[f].shape[0]] = meta[f]
+
+        dev = wrapper.begin_forward_with_metadata(
+            total, fill, starts["kv_page_indptr"], starts["kv_page_indices"], host["kv_page_indptr"],
+            host["kv_last_page_lens"], host["kv_page_indices"], num_qo_heads, num_kv_heads, head_dim,
+            page_size, pool.main_device, target_workgroups)
+        v = {f: dev[starts[f]: starts[f] + meta[f].shape[0]] for f in _FIELDS}
+        return cls(bsz=len(task_datas), seqlens=v["seqlens"], layer_id=0, page_pool=pool,
+                   offsets=v["offsets"], indptr=v["indptr"], kv_page_indices=v["kv_page_indices"],
+                   kv_page_indptr=v["kv_page_indptr"], kv_last_page_lens=v["kv_last_page_lens"],
+                   host=host, decode_wrapper=wrapper)
 
 
 @dataclass

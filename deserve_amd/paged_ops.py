@@ -164,9 +164,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         h_last = self._host(last_page_len, last_page_len_host)
         self._check_block_tables(h_indptr, indices, indices_host)
         batch = h_indptr.shape[0] - 1
-        L = _lib.lib()
-        total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
-        cap = L.dskv_decode_plan_bound(batch, total_tokens)
+        cap = self._plan_bound(batch, h_indptr, page_size)
         if plan_buffers is not None:
             if plan_buffers.dev.numel() < cap:
                 raise ValueError(f"plan buffer holds {plan_buffers.dev.numel()} words, {cap} may be needed")
@@ -174,23 +172,66 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         else:
             block = staging.take(max(cap, 1))
             plan = block.tensor
+        words = self._plan_into(plan, cap, h_indptr, h_last, target_workgroups)
+        if plan_buffers is not None:
+            self._plan = plan_buffers.dev
+            plan_buffers.upload(max(words, 1))
+        else:
+            self._plan = staging.to_device(block, max(words, 1), indices.device)
+        self._planned = True
+
+    @staticmethod
+    def _plan_bound(batch: int, h_indptr: torch.Tensor, page_size: int) -> int:
+        total_tokens = int(h_indptr[-1]) * page_size if batch > 0 else 0
+        return int(_lib.lib().dskv_decode_plan_bound(batch, total_tokens))
+
+    def _plan_into(self, plan: torch.Tensor, cap: int, h_indptr: torch.Tensor, h_last: torch.Tensor,
+                   target_workgroups: int) -> int:
+        """Runs the host planner into `plan` (pinned int32, at least cap words); returns the
+        words written.  Sets the launch shape of the following forward() calls."""
+        batch = h_indptr.shape[0] - 1
         n_items, n_wgs = ctypes.c_int32(), ctypes.c_int32()
         words, ws = ctypes.c_int64(), ctypes.c_int64()
-        rc = L.dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, page_size,
-                                num_qo_heads, num_kv_heads, head_dim, target_workgroups,
-                                plan.data_ptr(), cap, ctypes.byref(n_items), ctypes.byref(n_wgs),
-                                ctypes.byref(words), ctypes.byref(ws))
+        rc = _lib.lib().dskv_decode_plan(h_indptr.data_ptr(), h_last.data_ptr(), batch, self._p,
+                                         self._hq, self._hkv, self._d, target_workgroups,
+                                         plan.data_ptr(), cap, ctypes.byref(n_items), ctypes.byref(n_wgs),
+                                         ctypes.byref(words), ctypes.byref(ws))
         _lib.check(rc, "decode begin_forward")
         if ws.value > self._workspace.numel() * self._workspace.element_size():
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
         self._rope_table, self._rope_key = None, None     # positions change with the step
-        if plan_buffers is not None:
-            self._plan = plan_buffers.dev
-            plan_buffers.upload(max(words.value, 1))
-        else:
-            self._plan = staging.to_device(block, max(words.value, 1), indices.device)
+        return int(words.value)
+
+    def begin_forward_with_metadata(self, meta_words: int, fill_metadata, indptr_at: int, indices_at: int,
+                                    indptr_host: torch.Tensor, last_page_len_host: torch.Tensor,
+                                    indices_host: torch.Tensor, num_qo_heads: int, num_kv_heads: int,
+                                    head_dim: int, page_size: int, device: torch.device,
+                                    target_workgroups: int = 0) -> torch.Tensor:
+        """begin_forward for callers that also have the step's other index arrays to upload
+        (the forward context): metadata and work list travel in ONE pinned block and ONE
+        upload kernel instead of one each.  fill_metadata(view) writes the caller's
+        meta_words int32 words (a multiple of 4) into the front of the block; indptr_at /
+        indices_at are the word offsets of kv_page_indptr and kv_page_indices in it.  Returns
+        the device tensor that holds the metadata words (the caller slices its views)."""
+        if meta_words % 4:
+            raise ValueError("meta_words must be a multiple of 4 (16-byte alignment of the work list)")
+        self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
+        h_indptr = indptr_host.to(torch.int32).contiguous()
+        h_last = last_page_len_host.to(torch.int32).contiguous()
+        self._check_block_tables(h_indptr, indices_host, indices_host)
+        batch = h_indptr.shape[0] - 1
+        cap = self._plan_bound(batch, h_indptr, page_size)
+        block = staging.take(meta_words + max(cap, 4))
+        fill_metadata(block.tensor[:meta_words])
+        words = self._plan_into(block.tensor[meta_words:], cap, h_indptr, h_last, target_workgroups)
+        dev = staging.to_device(block, meta_words + max(words, 1), device)
+        self._plan = dev[meta_words:]
+        self._indptr = dev[indptr_at: indptr_at + batch + 1]
+        used = int(h_indptr[-1]) if batch > 0 else 0
+        self._indices = dev[indices_at: indices_at + used]
         self._planned = True
+        return dev[:meta_words]
 
     def fused_append_supported(self, dtype: torch.dtype) -> bool:
         """Whether forward(..., k_append=, v_append=) can write the step's token itself for

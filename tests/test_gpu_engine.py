@@ -302,6 +302,46 @@ def test_graphed_decode_step_matches_eager_steps():
     assert step.captures == 2 and len(step._graphs) == 2       # both batch shapes are held for replay
 
 
+def test_joined_prepare_equals_context_then_begin_forward():
+    """FlashDecodeCtx.init_and_plan (metadata and work list in one pinned block, one upload
+    kernel) against init_paged_decode_ctx + begin_forward (one upload each): the same six
+    arrays on the device, the same work list, the same launch shape, the same output bits."""
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.model.context.flash import FlashDecodeCtx
+    from deserve_amd.synthetic import make_decode_workload
+
+    print("[case] joined prepare", flush=True)
+    lens = np.array([13, 16, 300, 47, 1000, 31, 1, 4095])
+    fresh = lambda: make_decode_workload("j", lens, 2, HQ, HKV, D, P, torch.bfloat16, headroom_tokens=64,
+                                         seed=31, fill=True)
+    wl_a, wl_b = fresh(), fresh()
+    w_a, _ = get_wrappers(DEV)
+    w_b = type(w_a)(torch.empty(32 << 20, dtype=torch.uint8, device=DEV))
+    shape = dict(num_qo_heads=HQ, num_kv_heads=HKV, head_dim=D, page_size=P)
+    for step in range(3):                                   # lengths 16 and 4095 cross a page boundary
+        a = FlashDecodeCtx.init_paged_decode_ctx(wl_a.tasks, wl_a.caches, w_a)
+        w_a.begin_forward(indptr=a.kv_page_indptr, indices=a.kv_page_indices, last_page_len=a.kv_last_page_lens,
+                          indptr_host=a.host["kv_page_indptr"], last_page_len_host=a.host["kv_last_page_lens"],
+                          indices_host=a.host["kv_page_indices"], target_workgroups=24, **shape)
+        b = FlashDecodeCtx.init_and_plan(wl_b.tasks, wl_b.caches, w_b, target_workgroups=24, **shape)
+        for f in ("indptr", "kv_page_indices", "kv_page_indptr", "kv_last_page_lens", "offsets", "seqlens"):
+            assert torch.equal(getattr(a, f), getattr(b, f)), f
+            assert torch.equal(getattr(b, f).cpu(), b.host[f]), f
+        assert (w_a._n_items, w_a._n_workgroups, w_a._batch) == (w_b._n_items, w_b._n_workgroups, w_b._batch)
+        assert torch.equal(w_a._plan[: w_b._plan.numel()], w_b._plan[: w_a._plan.numel()])
+        assert torch.equal(w_b._indices, b.kv_page_indices) and torch.equal(w_b._indptr, b.kv_page_indptr)
+        for layer in range(2):
+            out_a = w_a.forward(wl_a.q[layer], wl_a.pool.pages[layer], k_append=wl_a.k[layer], v_append=wl_a.v[layer])
+            out_b = w_b.forward(wl_b.q[layer], wl_b.pool.pages[layer], k_append=wl_b.k[layer], v_append=wl_b.v[layer])
+            assert torch.equal(out_a.view(torch.int16), out_b.view(torch.int16)), (step, layer)
+        w_a.end_forward()
+        w_b.end_forward()
+        for wl in (wl_a, wl_b):
+            for t in wl.tasks:
+                t.step()
+    assert torch.equal(wl_a.pool.pages.view(torch.int16), wl_b.pool.pages.view(torch.int16))
+
+
 def test_graphed_decode_step_on_the_generic_kernel_follows_the_item_count():
     """head_dim 64 takes the generic attention kernel, which is launched with one workgroup
     per work item: a captured launch is only valid for its item count.  Contexts grow by a
