@@ -5,12 +5,15 @@
 // one tile of query rows; each of its waves owns 32 columns (kColTiles tiles of
 // 32), a column being a (query position, q head of the GQA group) pair, so the
 // MFMA N dimension is dense.  The workgroup walks the request's K/V in blocks of
-// 32 tokens that its waves load together (each a few rows) into LDS stages, so a
+// 32 tokens that its waves load together (each four rows) into LDS stages, so a
 // K/V byte crosses the vector memory path once per workgroup instead of once per
 // wave: with every wave streaming K/V on its own the kernel was bound by that
-// path at a sixth of the MFMA rate.  Row pitches of 272 (K) and 320 (V) bytes keep
-// the operand reads free of LDS bank conflicts (SQ_LDS_BANK_CONFLICT = 0; 288 for
-// either costs 4 %).
+// path at a sixth of the MFMA rate.  The rows go from global memory straight into
+// LDS (`buffer_load_dwordx4 ... lds`, three blocks ahead of their use), without a
+// trip through vector registers; pages shorter than four tokens take the register
+// path (load, then ds_write) instead.  The loads are inline assembly with hand-set
+// `s_waitcnt vmcnt` and a bare `s_barrier`: through the compiler's builtin every
+// barrier and LDS read waited for all loads in flight, which undid the prefetch.
 //
 // All products use the 32x32x16 MFMA (measured on MI355X at 2.2 PFLOP/s bf16,
 // against 1.3 PFLOP/s for 16x16x32).  Per block a wave computes S^T = K.Q^T
@@ -31,12 +34,6 @@ namespace dskv {
 #ifndef DSKV_PREFILL_WAVES
 #define DSKV_PREFILL_WAVES 8
 #endif
-#ifndef DSKV_PREFILL_KPITCH
-#define DSKV_PREFILL_KPITCH 272
-#endif
-#ifndef DSKV_PREFILL_VPITCH
-#define DSKV_PREFILL_VPITCH 320
-#endif
 #ifndef DSKV_PREFILL_COLTILES
 #define DSKV_PREFILL_COLTILES 1
 #endif
@@ -44,18 +41,22 @@ constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
 constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
 constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
 constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
-constexpr int kKPitch = DSKV_PREFILL_KPITCH;        // bytes per K row in LDS (256 + pad)
-constexpr int kPVPitch = DSKV_PREFILL_VPITCH;       // bytes per V row in LDS (256 + pad)
 constexpr int kRowsPerWave = kBlock / kPrefillWaves;   // rows of a block one wave loads
 constexpr int kRowGroups = kRowsPerWave / 4;           // in groups of 4 rows (one load each)
 static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole groups of 4 rows");
+// LDS layout of a 32-token block of K (or V) rows of one kv head: eight regions of four rows.
+// A region is what one load instruction delivers: 64 lanes x 16 bytes, lane p at byte 16 p.
+// Lane p = 4 c + rho fetches the 16-byte chunk c of row rho, so the region holds its rows
+// interleaved chunk by chunk ((4 c + rho) * 16); regions are 1088 bytes apart (64 bytes of
+// padding).  Operand reads are free of bank conflicts: the 16 lanes of a K-operand read (16
+// token rows, one chunk) and the 32 lanes of a transposing V read (4 rows x 4 chunks of a
+// region) fall on 16 different 16-byte bank groups each.
+constexpr int kRegionBytes = 1088;
+constexpr int kStageBytes = (kBlock / 4) * kRegionBytes;
 // The running maximum of a column is only raised when a block exceeds it by more
 // than this (log2 domain): probabilities stay below 2^8, the accumulators are
 // rescaled a handful of times per query instead of once per block.
 constexpr float kRescaleSlack = 8.f;
-#ifndef DSKV_PREFILL_LOOKUP_FIRST
-#define DSKV_PREFILL_LOOKUP_FIRST 1
-#endif
 #ifndef DSKV_PREFILL_KREADS_FIRST
 #define DSKV_PREFILL_KREADS_FIRST 0
 #endif
@@ -79,8 +80,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     int n_kv_heads, int page_shift, float scale_log2, int causal)
 {
     typedef Elt<DT> E;
-    __shared__ __align__(16) char k_stage[2][kBlock * kKPitch];
-    __shared__ __align__(16) char v_stage[4][kBlock * kPVPitch];
+    __shared__ __align__(16) char k_stage[4][kStageBytes];
+    __shared__ __align__(16) char v_stage[4][kStageBytes];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -180,29 +181,43 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         return;
     }
 
-    // This wave's share of the K (or V) rows of block blk: rows
-    // wave*kRowsPerWave .. +kRowsPerWave, lane (g, c) the 16-byte chunk c of row
-    // 4i + g.  Rows at or past t_end read as zero (their probabilities are zero,
-    // but 0 * garbage is not).  Page ids are looked up with a vector load (every
-    // lane the same entry; entries past the table read as page 0, whose
-    // descriptor is then empty): vector loads return in order, so waiting for an
-    // LDS read does not have to wait for these too, as it would for a scalar load.
-    const int lane_off = g * row_bytes + kvh * (kHeadDim * 2) + c * 16;
-    __amdgpu_buffer_rsrc_t page_table = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<int32_t *>(kv_indices + kv_indptr[b]), 0, n_pages * 4, kBufferFlags);
+    // This wave's share of the K (or V) rows of block blk: rows wave*kRowsPerWave .. +kRowsPerWave,
+    // in groups of four (one region each).  Rows at or past t_end arrive as zeros (their
+    // probabilities are zero, but 0 * garbage is not).
+    //
+    // Pages of at least four tokens (kRowsSharePage): the rows go from memory straight into
+    // their LDS region (buffer_load ... lds: lane p's 16 bytes land at region + 16 p, lanes
+    // beyond the descriptor's end write zeros), addressed through descriptors that end after
+    // the group's last valid row.  Page ids are looked up with a vector load (every lane the
+    // same entry; entries past the table read as page 0, whose descriptor is then empty).
+    // Smaller pages: every lane resolves its own page, the rows pass through registers.
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const int direct_off = (lane & 3) * row_bytes + kvh * (kHeadDim * 2) + (lane >> 2) * 16;
+    const int lane_off = kvh * (kHeadDim * 2) + c * 16;
+    // Page ids come through scalar loads (block-table entries past the table are clamped to
+    // its last one; their descriptors are empty).  They are consumed at the end of an
+    // iteration, when every LDS read of the iteration has been waited for anyway (scalar
+    // loads and LDS reads share a counter).
+    const int last_entry = max(n_pages - 1, 0);
     auto lookup_pages = [&](int blk, int(&pg)[kRowGroups]) {
         if (!kRowsSharePage) return;
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
             const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
-            pg[i] = __builtin_amdgcn_raw_buffer_load_b32(page_table, (tok0 >> page_shift) * 4 + lane * 0, 0, 0);
+            pg[i] = page_ids[min(tok0 >> page_shift, last_entry)];
         }
     };
     // The descriptors of the rows of block blk (scalar work: page id into an SGPR, base
     // address, valid bytes), prepared an iteration before the loads are issued so that it
     // runs in the shadow of that iteration's MFMAs.
     struct RowDesc {
-        __amdgpu_buffer_rsrc_t k[kRowGroups], v[kRowGroups];
+        u32x4 k[kRowGroups], v[kRowGroups];   // raw buffer descriptors: base, base >> 32, bytes, flags
+    };
+    auto make_desc = [&](const char *base, int bytes) {
+        const uint64_t a = (uint64_t)base;
+        return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu)),
+                     (uint32_t)__builtin_amdgcn_readfirstlane(bytes), (uint32_t)kBufferFlags};
     };
     auto prepare_rows = [&](int blk, const int(&pg)[kRowGroups], RowDesc &d) {
         if (!kRowsSharePage) return;
@@ -211,56 +226,62 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
             // one page holds the 4 rows: descriptors that end after the last
             // valid row make the bounds check free and keep offsets constant
+            // (the clamp is selected as a vector instruction: back to a scalar register, the
+            // descriptor words must live in SGPRs)
             const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
-            const long page = __builtin_amdgcn_readfirstlane(pg[i]);
-            char *first_row = const_cast<char *>(pages) + page * page_bytes +
-                              (long)(tok0 & page_mask) * row_bytes;
-            d.k[i] = __builtin_amdgcn_make_buffer_rsrc(first_row, 0, valid * row_bytes, kBufferFlags);
-            d.v[i] = __builtin_amdgcn_make_buffer_rsrc(first_row + half_bytes, 0, valid * row_bytes,
-                                                       kBufferFlags);
+            const char *first_row = pages + (long)pg[i] * page_bytes + (long)(tok0 & page_mask) * row_bytes;
+            d.k[i] = make_desc(first_row, valid * row_bytes);
+            d.v[i] = make_desc(first_row + half_bytes, valid * row_bytes);
         }
     };
-    auto load_rows = [&](int blk, const RowDesc &d, u32x4(&k_rows)[kRowGroups],
-                         u32x4(&v_rows)[kRowGroups]) {
+    auto region_of = [&](char *stage, int i) { return stage + (wave * kRowGroups + i) * kRegionBytes; };
+    // Written out as instructions: through the compiler's builtin every later LDS read waits
+    // for ALL of these loads (it cannot tell which region a read touches), which would undo
+    // requesting them three iterations early.  What it does not know it does not wait for:
+    // the waits for these loads are the explicit ones below.
+    auto load_direct = [&](const u32x4(&rows)[kRowGroups], char *stage) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
-            if (kRowsSharePage) {
-                k_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(d.k[i], lane_off, 0, kLoadCached);
-                v_rows[i] = __builtin_amdgcn_raw_buffer_load_b128(d.v[i], lane_off, 0, kLoadCached);
-            } else {
-                const int tok = blk * kBlock + wave * kRowsPerWave + 4 * i + g;
-                const int tc = min(tok, t_end - 1);
-                const char *p = pages + page_ids[tc >> page_shift] * page_bytes +
-                                (long)(tc & page_mask) * row_bytes + (lane_off - g * row_bytes);
-                const u32x4 z = {0, 0, 0, 0};
-                const u32x4 got_k = *reinterpret_cast<const u32x4 *>(p);
-                const u32x4 got_v = *reinterpret_cast<const u32x4 *>(p + half_bytes);
-                k_rows[i] = tok < t_end ? got_k : z;
-                v_rows[i] = tok < t_end ? got_v : z;
-            }
+            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_ptr)region_of(stage, i);
+            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                         :
+                         : "s"(lds_addr), "v"(direct_off), "s"(rows[i])
+                         : "memory");
         }
     };
-    auto store_rows = [&](char *st, int pitch, const u32x4(&rows)[kRowGroups]) {
+    auto load_rows = [&](int blk, u32x4(&k_rows)[kRowGroups], u32x4(&v_rows)[kRowGroups]) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
-            const int row = wave * kRowsPerWave + 4 * i + g;
-            *reinterpret_cast<u32x4 *>(st + row * pitch + c * 16) = rows[i];
+            const int tok = blk * kBlock + wave * kRowsPerWave + 4 * i + g;
+            const int tc = max(min(tok, t_end - 1), 0);
+            const char *p = pages + page_ids[tc >> page_shift] * page_bytes +
+                            (long)(tc & page_mask) * row_bytes + lane_off;
+            const u32x4 z = {0, 0, 0, 0};
+            const u32x4 got_k = *reinterpret_cast<const u32x4 *>(p);
+            const u32x4 got_v = *reinterpret_cast<const u32x4 *>(p + half_bytes);
+            k_rows[i] = tok < t_end ? got_k : z;
+            v_rows[i] = tok < t_end ? got_v : z;
         }
     };
+    auto store_rows = [&](char *stage, const u32x4(&rows)[kRowGroups]) {   // lane (g, c): chunk c of row g
+#pragma unroll
+        for (int i = 0; i < kRowGroups; i++)
+            *reinterpret_cast<u32x4 *>(region_of(stage, i) + (c * 4 + g) * 16) = rows[i];
+    };
+    // Waits until at most n of this wave's vector-memory operations are outstanding (the
+    // other counters of s_waitcnt left at "do not wait").
+#define DSKV_WAIT_VMEM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | 0x70 | 0xF00 | (((n) >> 4) << 14))
 
-    // S^T = K.Q^T of one block, unscaled: tokens 8i + 4h + j of column r in
-    // x[4i + j].  Registers 8s .. 8s+7, packed, are the B operand of the P.V MFMA
-    // for k-step s, which thereby fixes the tokens of that step's k slots:
-    // 16s + 4h + j in slots j, 16s + 8 + 4h + j in slots 4 + j.
     // Two score buffers that the iterations use in turn (S(m) is still being turned into
     // P(m) while S(m+1) is computed): the loop is unrolled with static phases, so which
     // buffer is which is known at compile time and no copy is needed.
     f32x16 xs[2][kColTiles];
     u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
     auto read_k_operands = [&](const char *kst) {
-        const char *k_rows = kst + r * kKPitch + h * 16;
+        // token r = row r & 3 of region r >> 2; chunk 2 ks + h
+        const char *k_rows = kst + (r >> 2) * kRegionBytes + h * 64 + (r & 3) * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 32);
+        for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 128);
     };
     auto scores = [&](int buf) {
 #pragma unroll
@@ -311,50 +332,54 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     // Iteration m of the main loop multiplies P(m-1) into V(m-1), turns S(m) into
     // P(m) and computes S(m+1), so that every MFMA of the iteration is independent
     // of its exponentials and the matrix and vector pipelines of a wave overlap.
-    // The rows of block m+4 are requested in iteration m (their page id was looked
-    // up in iteration m-2, their descriptors built in iteration m-1 behind its
-    // MFMAs) and written to LDS in iteration m+2: one iteration is shorter than a
-    // trip to memory.  K has two LDS stages and V four (V(j) is
-    // read three iterations after it is stored).  Per iteration one barrier: past
-    // it K(m+1) and V(m-1) are complete and the stages of K(m) and V(m-2) are free.
-    // Every wave runs every iteration (idle ones only move rows), so the barriers
-    // match.  The loop is unrolled by four so that all stage indices are static.
+    // Block j lives in K stage j % 4 and V stage j % 4.  Per iteration one barrier; every
+    // wave runs every iteration (idle ones only move rows), so the barriers match.  The loop
+    // is unrolled by four so that all stage indices are static.
+    //   Direct path: iteration m requests K(m+3) and V(m+2) behind its barrier (K(m+3)
+    //   replaces K(m-1), last read in iteration m-2; V(m+2) replaces V(m-2), last read in
+    //   iteration m-1).  K(m+1), which iteration m reads, went out two iterations earlier; a
+    //   wave makes sure that its own part of it has landed (at most 3 younger loads per row
+    //   group outstanding: V(m), K(m+2), V(m+1)) before it joins the barrier
+    //   that publishes the block.  The page of block j is looked up in iteration j-5 and its
+    //   descriptors are built in iteration j-4, behind that iteration's MFMAs.
+    //   Register path: the rows of block m+4 are requested in iteration m and written to
+    //   LDS in iteration m+2 (one iteration is shorter than a trip to memory).
+    RowDesc desc[4];              // descriptors of block j in desc[j % 4]
+    int pg[4][kRowGroups];        // page ids of block j in pg[j % 4]
     struct RowSet {
-        u32x4 k[kRowGroups], v[kRowGroups];   // rows on their way to LDS
-        int pg[kRowGroups];                   // page ids of the rows requested next
-        RowDesc desc;                         // their descriptors, once prepared
+        u32x4 k[kRowGroups], v[kRowGroups];   // rows on their way to LDS (register path)
     };
     RowSet even, odd;
     {
-        int pg[kRowGroups];
-        u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
-#pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-            RowDesc d;
-            lookup_pages(blk, pg);
-            prepare_rows(blk, pg, d);
-            load_rows(blk, d, first_k[blk], first_v[blk]);
-        }
-        lookup_pages(2, even.pg);
-        lookup_pages(3, odd.pg);
         const u32x4 z = {0, 0, 0, 0};
         u32x4 zero[kRowGroups];
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) zero[i] = z;
-        store_rows(v_stage[3], kPVPitch, zero);   // V(-1): multiplied by P(-1) = 0, must be finite
+        store_rows(v_stage[3], zero);   // V(-1): multiplied by P(-1) = 0, must be finite
+        if (kRowsSharePage) {
 #pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-            store_rows(k_stage[blk], kKPitch, first_k[blk]);
-            store_rows(v_stage[blk], kPVPitch, first_v[blk]);
+            for (int blk = 0; blk < 4; blk++) lookup_pages(blk, pg[blk]);
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++) prepare_rows(blk, pg[blk], desc[blk]);
+#pragma unroll
+            for (int blk = 0; blk < 3; blk++) load_direct(desc[blk].k, k_stage[blk]);
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) load_direct(desc[blk].v, v_stage[blk]);
+            lookup_pages(4, pg[0]);
+            DSKV_WAIT_VMEM(0);
+        } else {
+            u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) load_rows(blk, first_k[blk], first_v[blk]);
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                store_rows(k_stage[blk], first_k[blk]);
+                store_rows(v_stage[blk], first_v[blk]);
+            }
+            load_rows(2, even.k, even.v);
+            load_rows(3, odd.k, odd.v);
         }
     }
-    prepare_rows(2, even.pg, even.desc);
-    prepare_rows(3, odd.pg, odd.desc);
-    load_rows(2, even.desc, even.k, even.v);
-    load_rows(3, odd.desc, odd.k, odd.v);
-    lookup_pages(4, even.pg);
-    lookup_pages(5, odd.pg);
-    prepare_rows(4, even.pg, even.desc);   // iteration 0 issues these; every iteration prepares the next one's
     __syncthreads();
     if (w_end > 0) {
         read_k_operands(k_stage[0]);
@@ -362,22 +387,32 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         if (kBlock > w_mask_from) mask_scores(0, 0);
         block_max(0);
     }
-    const int v_lane_off = (4 * h + (c >> 2)) * kPVPitch + (g & 1) * 32 + (c & 3) * 8;
-    auto iteration = [&](int m, int phase, RowSet &rows, RowSet &next) {   // phase = m % 4, a literal at each call
-        __syncthreads();
-        store_rows(k_stage[phase & 1], kKPitch, rows.k);              // K(m+2)
-        store_rows(v_stage[(phase + 2) & 3], kPVPitch, rows.v);       // V(m+2)
-#if DSKV_PREFILL_LOOKUP_FIRST
-        // the page lookup goes out before the row loads: vector loads return in order, so the
-        // wait for this lookup (next iteration) then leaves the row loads behind it in flight
-        lookup_pages(m + 6, rows.pg);
-        load_rows(m + 4, rows.desc, rows.k, rows.v);
-#else
-        load_rows(m + 4, rows.desc, rows.k, rows.v);
-        lookup_pages(m + 6, rows.pg);
-#endif
+    // V operand: token 16 ks + 8 hi + 4 h + (c >> 2) = row c >> 2 of region 4 ks + 2 hi + h;
+    // bytes 64 dt + 32 (g & 1) + 8 (c & 3) of its row = half (c & 1) of chunk 4 dt + 2 (g & 1) + ((c & 3) >> 1)
+    const int v_lane_off = h * kRegionBytes + (2 * (g & 1) + ((c & 3) >> 1)) * 64 + (c >> 2) * 16 + (c & 1) * 8;
+    auto iteration = [&](int m, int phase, RowSet &rows) {   // phase = m % 4, a literal at each call
+        if (kRowsSharePage) {
+            // this wave's rows of K(m+1) have landed; then the bare barrier: with the fences of
+            // __syncthreads the compiler waits for EVERY load into LDS still on its way, which
+            // is the whole point of requesting them early.  Nothing else needs the fences here:
+            // the loop of this path writes LDS through these loads only, and the LDS reads of
+            // the previous iteration have been consumed.
+            DSKV_WAIT_VMEM(3 * kRowGroups);
+            __builtin_amdgcn_s_barrier();
+        } else {
+            __syncthreads();
+        }
+        if (kRowsSharePage) {
+            lookup_pages(m + 5, pg[(phase + 1) & 3]);
+            load_direct(desc[(phase + 3) & 3].k, k_stage[(phase + 3) & 3]);   // K(m+3)
+            load_direct(desc[(phase + 2) & 3].v, v_stage[(phase + 2) & 3]);   // V(m+2)
+        } else {
+            store_rows(k_stage[(phase + 2) & 3], rows.k);                     // K(m+2)
+            store_rows(v_stage[(phase + 2) & 3], rows.v);                     // V(m+2)
+            load_rows(m + 4, rows.k, rows.v);
+        }
         if (!(w_end > 0 && (m - 1) * kBlock < w_end)) {
-            prepare_rows(m + 5, next.pg, next.desc);
+            prepare_rows(m + 4, pg[phase], desc[phase]);
             return;
         }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
@@ -420,7 +455,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         // V operand: the transposing read hands each block of 16 lanes four tokens
         // of 16 consecutive dims, lane i of the block supplying the address of dims
         // 4*(i%4) .. +3 of the block's token i/4
-        read_k_operands(k_stage[(phase + 1) & 1]);                       // K(m+1)
+        read_k_operands(k_stage[(phase + 1) & 3]);                       // K(m+1)
 #if DSKV_PREFILL_KREADS_FIRST
         __builtin_amdgcn_sched_barrier(0);   // all eight K operands requested before anything else
 #endif
@@ -430,9 +465,9 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const char *vp = v_rows + ks * 16 * kPVPitch + dt * 64;
+                const char *vp = v_rows + ks * 4 * kRegionBytes + dt * 256;
                 const u32x2 a_lo = read_transposed(vp);
-                const u32x2 a_hi = read_transposed(vp + 8 * kPVPitch);
+                const u32x2 a_hi = read_transposed(vp + 2 * kRegionBytes);
                 va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
             }
         scores(nxt);
@@ -467,17 +502,19 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ct++)
                     l_acc[ct] = E::mfma_32x32(ones, pb_prev[ct][ks], l_acc[ct]);
-        prepare_rows(m + 5, next.pg, next.desc);   // for the loads of the next iteration
+        prepare_rows(m + 4, pg[phase], desc[phase]);   // for the loads of the next iterations
         block_max(nxt);
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
     };
     for (int m = 0; m <= n_blocks; m += 4) {
-        iteration(m, 0, even, odd);
-        iteration(m + 1, 1, odd, even);
-        iteration(m + 2, 2, even, odd);
-        iteration(m + 3, 3, odd, even);
+        iteration(m, 0, even);
+        iteration(m + 1, 1, odd);
+        iteration(m + 2, 2, even);
+        iteration(m + 3, 3, odd);
     }
+    if (kRowsSharePage) DSKV_WAIT_VMEM(0);   // nothing of this wave may still be on its way into LDS
+#undef DSKV_WAIT_VMEM
 
 #pragma unroll
     for (int ct = 0; ct < kColTiles; ct++) {
