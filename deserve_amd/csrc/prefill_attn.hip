@@ -239,6 +239,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     // for ALL of these loads (it cannot tell which region a read touches), which would undo
     // requesting them three iterations early.  What it does not know it does not wait for:
     // the waits for these loads are the explicit ones below.
+    // M0 is on the clobber list (the compiler reserves it, sets it itself before the few
+    // instructions that read it, and must not assume that such a setting survives this one).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
     auto load_direct = [&](const u32x4(&rows)[kRowGroups], char *stage) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
@@ -246,9 +250,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                          :
                          : "s"(lds_addr), "v"(direct_off), "s"(rows[i])
-                         : "memory");
+                         : "memory", "m0");
         }
     };
+#pragma clang diagnostic pop
     auto load_rows = [&](int blk, u32x4(&k_rows)[kRowGroups], u32x4(&v_rows)[kRowGroups]) {
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) {
