@@ -107,14 +107,23 @@ class _PagedWrapper:
         return src.to(torch.int32).contiguous()
 
     def _check_block_tables(self, h_indptr: torch.Tensor, indices: torch.Tensor,
-                            indices_host: Optional[torch.Tensor]) -> None:
+                            indices_host: Optional[torch.Tensor], h_last: torch.Tensor) -> None:
         """The kernels index the pool by block-table entries: refuse, on the host, tables that
-        are shorter than indptr says or hold a negative id, and remember the largest id so
-        that forward() can refuse a pool that does not have that page."""
+        are shorter than indptr says or hold a negative id, last-page lengths that are missing
+        or outside [1, page_size], and remember the largest id so that forward() can refuse a
+        pool that does not have that page."""
         batch = h_indptr.shape[0] - 1
         used = int(h_indptr[-1]) if batch > 0 else 0
         if batch > 0 and (int(h_indptr[0]) != 0 or bool((h_indptr[1:] < h_indptr[:-1]).any())):
             raise ValueError("kv page indptr must start at 0 and not decrease")
+        if h_last.numel() < max(batch, 0):
+            raise ValueError(f"kv last-page lengths hold {h_last.numel()} entries for {batch} requests")
+        if batch > 0:
+            last = h_last[:batch]
+            bad = (h_indptr[1:] > h_indptr[:-1]) & ((last < 1) | (last > self._p))
+            if bool(bad.any()):
+                b = int(bad.nonzero()[0])
+                raise ValueError(f"kv_last_page_len[{b}] = {int(last[b])} outside [1, {self._p}]")
         if indices.numel() < used:
             raise ValueError(f"kv page indices hold {indices.numel()} entries, indptr[-1] is {used}")
         ids = self._host(indices, indices_host)[:used]
@@ -162,7 +171,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         self._indptr, self._indices = _i32(indptr), _i32(indices)
         h_indptr = self._host(indptr, indptr_host)
         h_last = self._host(last_page_len, last_page_len_host)
-        self._check_block_tables(h_indptr, indices, indices_host)
+        self._check_block_tables(h_indptr, indices, indices_host, h_last)
         batch = h_indptr.shape[0] - 1
         cap = self._plan_bound(batch, h_indptr, page_size)
         if plan_buffers is not None:
@@ -219,7 +228,7 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         h_indptr = indptr_host.to(torch.int32).contiguous()
         h_last = last_page_len_host.to(torch.int32).contiguous()
-        self._check_block_tables(h_indptr, indices_host, indices_host)
+        self._check_block_tables(h_indptr, indices_host, indices_host, h_last)
         batch = h_indptr.shape[0] - 1
         cap = self._plan_bound(batch, h_indptr, page_size)
         block = staging.take(meta_words + max(cap, 4))
@@ -330,7 +339,8 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         h_kv = self._host(paged_kv_indptr, paged_kv_indptr_host)
         if h_kv.shape[0] != h_qo.shape[0]:
             raise ValueError("qo_indptr and paged_kv_indptr disagree about the batch")
-        self._check_block_tables(h_kv, paged_kv_indices, paged_kv_indices_host)
+        h_last32 = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host)
+        self._check_block_tables(h_kv, paged_kv_indices, paged_kv_indices_host, h_last32)
         L = _lib.lib()
         cap = L.dskv_prefill_plan_bound(batch, nnz)
         block = staging.take(max(cap, 2))
@@ -338,7 +348,7 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         n_tiles = ctypes.c_int32()
         # kv lengths order the tiles longest first
         h_indptr = h_kv.to(torch.int64)
-        h_last = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host).to(torch.int64)
+        h_last = h_last32.to(torch.int64)
         n_pages = h_indptr[1:] - h_indptr[:-1]
         kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
         rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,

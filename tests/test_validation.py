@@ -31,12 +31,16 @@ def test_decode_begin_forward_refuses_bad_block_tables():
     with pytest.raises(ValueError, match="indices_host holds 1"):
         _decode().begin_forward(_i32([0, 1, 3]), _i32([5, 6, 7]), _i32([16, 4]), indices_host=_i32([5]),
                                 indptr_host=_i32([0, 1, 3]), last_page_len_host=_i32([16, 4]), **shape)
+    with pytest.raises(ValueError, match="1 entries for 2 requests"):
+        _decode().begin_forward(_i32([0, 1, 3]), _i32([5, 6, 7]), _i32([16]), **shape)
+    with pytest.raises(ValueError, match="kv_last_page_len\\[1\\] = 17 outside \\[1, 16\\]"):
+        _decode().begin_forward(_i32([0, 1, 3]), _i32([5, 6, 7]), _i32([16, 17]), **shape)
 
 
 def test_forward_refuses_a_pool_that_lacks_a_named_page_or_has_another_shape():
     w = _decode()
     w._shape_args(32, 8, 128, 16)
-    w._check_block_tables(_i32([0, 1, 3]), _i32([5, 40, 7]), None)
+    w._check_block_tables(_i32([0, 1, 3]), _i32([5, 40, 7]), None, _i32([16, 4]))
     assert w._max_page_id == 40
     ok = torch.empty((41, 2, 16, 8, 128), dtype=torch.bfloat16)
     w._check_pool(ok, torch.bfloat16)
@@ -63,6 +67,10 @@ def test_prefill_begin_forward_refuses_bad_block_tables():
         w.begin_forward(_i32([0, 4, 8]), _i32([0, 1, 2]), _i32([3]), _i32([4, 4]), **shape)
     with pytest.raises(ValueError, match="qo_indptr"):
         w.begin_forward(_i32([0, 4, 2]), _i32([0, 1, 2]), _i32([3, 4]), _i32([4, 4]), **shape)
+    with pytest.raises(ValueError, match="kv_last_page_len\\[0\\] = 0 outside"):
+        w.begin_forward(_i32([0, 4, 8]), _i32([0, 1, 2]), _i32([3, 4]), _i32([0, 4]), **shape)
+    with pytest.raises(ValueError, match="1 entries for 2 requests"):
+        w.begin_forward(_i32([0, 4, 8]), _i32([0, 1, 2]), _i32([3, 4]), _i32([4]), **shape)
 
 
 def test_gather_and_scatter_refuse_page_ids_outside_the_pool():
