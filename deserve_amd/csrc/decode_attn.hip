@@ -79,13 +79,17 @@ struct LoadCursor {
     int next_item, item_end;   // next item to enter, one past the workgroup's last
     int t, t_end, t_pad_end;   // next tile, valid end and padded end of the current item
     const_i32_ptr page_ids;    // current item's block table
-    long page;                 // pool page of tile t, fetched one tile ahead of its use
+    long page[2];              // pool pages of tile t (one or two), fetched one tile ahead of their use
 };
 
 #ifndef DSKV_DECODE_MIN_WAVES
 #define DSKV_DECODE_MIN_WAVES 1
 #endif
-template <int DT, bool kPageCoversTile>
+// kPagesPerTile: pages a 16-token tile spans - 1 (pages of 16 tokens or more: one buffer
+// descriptor per tile), 2 (pages of 8 tokens: the two page ids as scalars, selected per
+// lane), 0 (smaller pages: every lane looks its page up itself; with four scalar ids and a
+// four-way selection pages of 4 tokens were slower than that, 130 against 113 us).
+template <int DT, int kPagesPerTile>   // 1, 2 or 0
 __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_attn_mfma_kernel(
     uint16_t *__restrict__ out, const uint16_t *__restrict__ q, const char *pages,
     const int32_t *__restrict__ kv_indices, const Item *__restrict__ items,
@@ -95,6 +99,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     const float *__restrict__ rope)
 {
     typedef Elt<DT> E;
+    constexpr bool kPageCoversTile = kPagesPerTile == 1;
     __shared__ __align__(16) char v_lds[kMaxWaves][kVTileBytes];
 
     const int wave = threadIdx.x >> 6;
@@ -203,10 +208,18 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     cur.item_end = item_end;
     cur.t = cur.t_end = cur.t_pad_end = 0;
     cur.page_ids = indices_c;
-    cur.page = 0;
+    for (long &pg : cur.page) pg = 0;
     auto fetch_page = [&]() {
         kv.page_ids = cur.page_ids;
-        if (kPageCoversTile) cur.page = cur.page_ids[page_slot_of(kv, cur.t, cur.t_end)];
+        if (kPageCoversTile) cur.page[0] = cur.page_ids[page_slot_of(kv, cur.t, cur.t_end)];
+        if (kPagesPerTile > 1) {
+            // an exhausted stream (t_end == 0) keeps loading from page 0, which every pool has
+#pragma unroll
+            for (int j = 0; j < kPagesPerTile; j++)
+                cur.page[j] = cur.t_end > 0
+                                  ? cur.page_ids[page_slot_of(kv, cur.t + (j << kv.page_shift), cur.t_end)]
+                                  : 0;
+        }
     };
     auto settle = [&]() {   // step into following items until a tile is available (or none is left)
         while (cur.t >= cur.t_pad_end && cur.next_item < cur.item_end) {
@@ -221,8 +234,17 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     };
     auto load_next = [&](TileRegs &r) {
         kv.page_ids = cur.page_ids;
-        if (kPageCoversTile) load_kv_tile_in_page<kLoadStreaming>(kv, cur.page, cur.t, cur.t_end, g, c, r);
-        else load_kv_tile<false, kLoadStreaming>(kv, cur.t, cur.t_end, g, c, r);
+        if (kPageCoversTile) {
+            load_kv_tile_in_page<kLoadStreaming>(kv, cur.page[0], cur.t, cur.t_end, g, c, r);
+        } else if (kPagesPerTile > 1) {
+            long pages_of_tile[kPagesPerTile > 1 ? kPagesPerTile : 1];
+#pragma unroll
+            for (int j = 0; j < kPagesPerTile; j++) pages_of_tile[j] = cur.page[j];
+            load_kv_tile_small_pages<(kPagesPerTile > 1 ? kPagesPerTile : 1), kLoadStreaming>(
+                kv, pages_of_tile, cur.t, cur.t_end, g, c, r);
+        } else {
+            load_kv_tile<false, kLoadStreaming>(kv, cur.t, cur.t_end, g, c, r);
+        }
         cur.t += kTile;
         settle();
     };
@@ -717,11 +739,13 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
                        wg_ptr, part_o, part_ml, (int)max_slots, n_qo_heads, n_kv_heads, shift,   \
                        scale_log2, (const uint16_t *)k_new, (const uint16_t *)v_new, rope_table)
         if (dtype == DSKV_BF16) {
-            if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_BF16, true);
-            else DSKV_LAUNCH_MFMA(DSKV_BF16, false);
+            if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_BF16, 1);
+            else if (page_size == 8) DSKV_LAUNCH_MFMA(DSKV_BF16, 2);
+            else DSKV_LAUNCH_MFMA(DSKV_BF16, 0);
         } else {
-            if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_F16, true);
-            else DSKV_LAUNCH_MFMA(DSKV_F16, false);
+            if (page_size >= kTile) DSKV_LAUNCH_MFMA(DSKV_F16, 1);
+            else if (page_size == 8) DSKV_LAUNCH_MFMA(DSKV_F16, 2);
+            else DSKV_LAUNCH_MFMA(DSKV_F16, 0);
         }
 #undef DSKV_LAUNCH_MFMA
         DSKV_LAUNCH_CHECK("decode_attn_mfma_kernel");

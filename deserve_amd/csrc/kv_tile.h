@@ -121,6 +121,40 @@ __device__ __forceinline__ void load_kv_tile(const KvView &kv, int t, int t_end,
     }
 }
 
+// Loads tile [t, t + 16) when a page holds fewer tokens than a tile (kPages pages per tile;
+// used for pages of 8 tokens, kPages = 2).  The tile's page ids come in as scalars (looked up one
+// tile ahead with scalar loads, like the single page of the path above); every lane selects
+// the page of its row among them.  Looking the ids up per lane with vector loads instead
+// would put a dependent load in front of every tile, and since a wave's vector loads return
+// in order, waiting for it means waiting for every tile still in flight: with pages of 8
+// tokens the pass took 114 us; this way 100 (98 with pages of 16).  Tokens past the end are clamped to the last
+// valid one, as in the per-lane path; page[0] is a valid page of the request also for a tile
+// that lies wholly past the end.
+template <int kPages, int kAux>
+__device__ __forceinline__ void load_kv_tile_small_pages(const KvView &kv, const long (&page)[kPages],
+                                                         int t, int t_end, int g, int c, TileRegs &r)
+{
+    const int page_mask = (1 << kv.page_shift) - 1;
+    const int t_last = max(t_end - 1, 0);
+    auto row_of = [&](int tok) -> const char * {
+        const int tc = min(tok, t_last);
+        const int j = max(tc - t, 0) >> kv.page_shift;
+        long pg = page[0];
+#pragma unroll
+        for (int i = 1; i < kPages; i++) pg = j == i ? page[i] : pg;
+        return kv.pages + pg * kv.page_bytes + (long)(tc & page_mask) * kv.row_bytes + kv.head_off;
+    };
+    auto load16 = [](const char *p) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(p);
+        return kAux == kLoadStreaming ? __builtin_nontemporal_load(q) : *q;
+    };
+    const char *kp = row_of(t + c) + g * 16;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) r.k[kk] = load16(kp + kk * 64);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.v[i] = load16(row_of(t + g + 4 * i) + kv.half_bytes + c * 16);
+}
+
 // V tile -> this wave's LDS tile.  Rows at or past t_end must be zero (their
 // probabilities are zero, but 0 * garbage is not): the buffer-descriptor path
 // already delivers zeros, the clamped path zeroes them here.  The tile is

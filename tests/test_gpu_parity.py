@@ -128,6 +128,10 @@ DECODE_CASES = [
     ("page8", [1000, 64, 333, 7, 8, 9], 8, 32, 8, 128, "bf16", 16),
     ("page4", [100, 3, 19], 4, 32, 8, 128, "f16", 4),
     ("page32", [1000, 31, 33, 64], 32, 32, 8, 128, "bf16", 16),
+    ("page8_long", [5000, 2100, 17, 8, 1], 8, 32, 8, 128, "bf16", 0),   # two pages per tile, default plan
+    ("page4_long", [3000, 5, 4, 1023], 4, 64, 8, 128, "f16", 0),       # four pages per tile
+    ("page2", [70, 5, 33], 2, 32, 8, 128, "bf16", 4),                   # per-lane page lookup
+    ("page1", [40, 3], 1, 32, 8, 128, "f16", 0),
     ("mha", [300, 40], 16, 8, 8, 128, "bf16", 0),
     ("group16", [300, 40], 16, 32, 2, 128, "bf16", 8),
     ("kv4", [300, 40, 1], 16, 16, 4, 128, "bf16", 0),
