@@ -389,6 +389,44 @@ def prefill_section(seed: int):
     attn_zero_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
     w.end_forward()
     append_bytes = 2 * B * n * 2 * Hkv * D * 2
+
+    # One 512-token chunk over 4096 prior tokens: the step budget of the reference's scheduler
+    # (engine/pipeline/scheduler.py:74,85).  8 query tiles x 8 kv heads are 64 workgroups, so
+    # the plan cuts every tile's K/V range into parts (merged by a second pass); timed with
+    # that plan and with whole tiles.
+    one_prior = 4096
+    one_pool = GpuPagePool(2, (one_prior + n) // P + 8, P, dev, torch.bfloat16)
+    fill_normal(one_pool.pages, seed + 44)
+    one_rows = PageTableAllocator(1, one_prior + 1024, P, dev)
+    one_task = [TaskData("p_one", one_prior, 1, n, one_prior + n, SamplingParams())]
+    one_cache = [PagedKVCache.empty(one_rows, one_pool)]
+    one_w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+    one_c = FlashPrefillCtx.init_paged_prefill_ctx(one_task, one_cache, one_w)
+    one_q = torch.randn((2, n, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
+    one_chunk = {}
+    for label, target in (("parts", 0), ("whole_tiles", -1)):
+        one_w.begin_forward(qo_indptr=one_c.indptr, paged_kv_indptr=one_c.kv_page_indptr,
+                            paged_kv_indices=one_c.kv_page_indices,
+                            paged_kv_last_page_len=one_c.kv_last_page_lens, num_qo_heads=Hq,
+                            num_kv_heads=Hkv, head_dim=D, page_size=P, qo_indptr_host=one_c.host["indptr"],
+                            paged_kv_indptr_host=one_c.host["kv_page_indptr"],
+                            paged_kv_last_page_len_host=one_c.host["kv_last_page_lens"],
+                            paged_kv_indices_host=one_c.host["kv_page_indices"], target_workgroups=target)
+        evs = []
+        for rep in range(12):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            one_w.forward(one_q[rep % 2], one_pool.pages[rep % 2], causal=True)
+            e.record()
+            evs.append((s, e))
+        torch.cuda.synchronize()
+        ts = sorted(s.elapsed_time(e) for s, e in evs[2:])
+        one_chunk[label] = {"parts_per_tile": one_w._n_splits, "workgroups": one_w._n_tiles * Hkv,
+                            "us_per_layer": round(ts[len(ts) // 2] * 1e3, 1)}
+        one_w.end_forward()
+    one_flops = 4 * Hq * D * (n * one_prior + n * (n + 1) // 2)
+    for v in one_chunk.values():
+        v["TFLOPs"] = round(one_flops / v["us_per_layer"] / 1e6, 1)
     return {"workload": "BASELINE.json configs[3]: bf16, GQA 32q/8kv, page 16, 16 sequences x 512-token "
                         "chunk appended at offsets U[0,15], attention over prior U[0,8192]; per layer",
             "chunk_tokens": B * n, "kv_tokens": int((prior + n).sum()),
@@ -399,7 +437,8 @@ def prefill_section(seed: int):
             "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
             "attention_us_per_layer_zero_data": round(attn_zero_us, 1),
             "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
-            "flops_per_layer": flops}
+            "flops_per_layer": flops,
+            "one_512_token_chunk_over_4096": one_chunk}
 
 
 def fragmented_section(seed: int):

@@ -56,11 +56,13 @@ _SIGNATURES = {
                                                c_int64, c_int32, c_int32, c_int32, c_int32, c_int32,
                                                c_float, c_int32, c_void_p, c_int32, c_void_p]),
     "dskv_prefill_plan_bound": (c_int64, [c_int32, c_int64]),
-    "dskv_prefill_plan": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_int64,
-                                    POINTER(c_int32)]),
+    "dskv_prefill_plan": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
+                                    c_void_p, c_int64, POINTER(c_int32), POINTER(c_int32),
+                                    POINTER(c_int64), POINTER(c_int64)]),
     "dskv_prefill_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                    c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32,
-                                    c_int32, c_int32, c_float, c_int32, c_int32, c_void_p]),
+                                    c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_int64, c_int32,
+                                    c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
+                                    c_int32, c_void_p]),
     "dskv_apply_rope": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
                                   c_void_p]),

@@ -45,6 +45,17 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+// Merge pass over per-part partials (max, sum, unnormalised O) in a workspace laid out as
+// [max_slots x n_qo_heads x head_dim] floats of O followed by [max_slots x n_qo_heads x 2] of
+// (max, sum): row r of `out` (rows x n_qo_heads x head_dim, of `dtype`) is merged from the
+// row_parts[2r + 1] parts that start at slot row_parts[2r]; rows with no parts are left
+// alone.  `wide`: eight waves per (row, head), for rows cut into dozens of parts.  Defined
+// beside the decode attention kernels, which write such partials; the prefill attention
+// kernel writes them too when its plan splits tiles.
+int launch_partials_merge(void *out, const float *part_o, const float *part_ml,
+                          const int32_t *row_parts, int max_slots, int rows, int n_qo_heads,
+                          int head_dim, int dtype, bool wide, hipStream_t stream);
+
 static inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 static inline int ilog2(int64_t x) {
     int s = 0;

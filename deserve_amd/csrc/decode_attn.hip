@@ -762,26 +762,35 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
         DSKV_LAUNCH_CHECK("decode_attn_generic_kernel");
     }
     if ((phases & 2) && n_items > batch) {
-        dim3 grid((unsigned)batch, (unsigned)n_qo_heads);
         // many parts per request (long requests, small batch): eight waves share a merge.
         // One wave needs a round trip per 8 parts, eight waves a barrier and a second pass
         // through LDS: they break even at about 32 parts.
         const bool wide = (int64_t)n_items > 32 * (int64_t)batch;
+        return launch_partials_merge(out, part_o, part_ml, req_parts, (int)max_slots, batch, n_qo_heads,
+                                     head_dim, dtype, wide, s);
+    }
+    return 0;
+}
+
+int launch_partials_merge(void *out, const float *part_o, const float *part_ml,
+                          const int32_t *row_parts, int max_slots, int rows, int n_qo_heads,
+                          int head_dim, int dtype, bool wide, hipStream_t s)
+{
+    dim3 grid((unsigned)rows, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_MERGE(DT)                                                                     \
     do {                                                                                          \
         if (wide)                                                                                 \
             hipLaunchKernelGGL((decode_merge_kernel<DT, 8>), grid, dim3(512), 0, s, out, part_o,  \
-                               part_ml, req_parts, (int)max_slots, n_qo_heads, head_dim);         \
+                               part_ml, row_parts, max_slots, n_qo_heads, head_dim);              \
         else                                                                                      \
             hipLaunchKernelGGL((decode_merge_kernel<DT, 1>), grid, dim3(64), 0, s, out, part_o,   \
-                               part_ml, req_parts, (int)max_slots, n_qo_heads, head_dim);         \
+                               part_ml, row_parts, max_slots, n_qo_heads, head_dim);              \
     } while (0)
-        if (dtype == DSKV_F32) DSKV_LAUNCH_MERGE(DSKV_F32);
-        else if (dtype == DSKV_F16) DSKV_LAUNCH_MERGE(DSKV_F16);
-        else DSKV_LAUNCH_MERGE(DSKV_BF16);
+    if (dtype == DSKV_F32) DSKV_LAUNCH_MERGE(DSKV_F32);
+    else if (dtype == DSKV_F16) DSKV_LAUNCH_MERGE(DSKV_F16);
+    else DSKV_LAUNCH_MERGE(DSKV_BF16);
 #undef DSKV_LAUNCH_MERGE
-        DSKV_LAUNCH_CHECK("decode_merge_kernel");
-    }
+    DSKV_LAUNCH_CHECK("decode_merge_kernel");
     return 0;
 }
 

@@ -41,6 +41,7 @@ constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
 constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
 constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
 constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
+constexpr int kTileWords = 5;                       // plan entry: request, first row, block range, part
 constexpr int kRowsPerWave = kBlock / kPrefillWaves;   // rows of a block one wave loads
 constexpr int kRowGroups = kRowsPerWave / 4;           // in groups of 4 rows (one load each)
 static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole groups of 4 rows");
@@ -77,7 +78,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
     const int32_t *__restrict__ kv_indices, const int32_t *__restrict__ kv_indptr,
     const int32_t *__restrict__ kv_last, const int32_t *__restrict__ tile_info, int n_qo_heads,
-    int n_kv_heads, int page_shift, float scale_log2, int causal)
+    int n_kv_heads, int page_shift, float scale_log2, int causal, int n_splits,
+    float *__restrict__ part_o, float *__restrict__ part_ml, int max_slots)
 {
     typedef Elt<DT> E;
     __shared__ __align__(16) char k_stage[4][kStageBytes];
@@ -94,12 +96,21 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const int group = n_qo_heads / n_kv_heads;
     const int pos_per_wave = kWaveCols / group;    // query positions per wave
 
-    const int b = tile_info[2 * tile];
-    const int q0 = tile_info[2 * tile + 1];        // first query row of the tile within b
+    // plan entry: request, first query row of the tile within it, and the 32-token blocks
+    // [blk_begin, blk_end) of the request's K/V that this workgroup walks (all of them unless
+    // the plan splits tiles; blk_begin is a multiple of four), as part `split` of n_splits
+    const const_i32_ptr entry = as_const(tile_info) + (long)tile * kTileWords;
+    const int b = entry[0];
+    const int q0 = entry[1];
+    const int blk_begin = entry[2];
+    const int kv_cap_blocks = entry[3];
+    const int split = entry[4];
     const int q_begin = qo_indptr[b];
     const int n_b = qo_indptr[b + 1] - q_begin;
     const int n_pages = kv_indptr[b + 1] - kv_indptr[b];
     const int kv_len = n_pages > 0 ? ((n_pages - 1) << page_shift) + kv_last[b] : 0;
+    // tokens this workgroup may look at end here: the request's end, or the end of its part
+    const int kv_cap = min(kv_len, kv_cap_blocks < (1 << 25) ? kv_cap_blocks * kBlock : kv_len);
     const_i32_ptr page_ids = as_const(kv_indices) + kv_indptr[b];
     const int row_bytes = n_kv_heads * kHeadDim * 2;
     const int half_bytes = row_bytes << page_shift;
@@ -119,7 +130,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
         qrow[ct] = wq0 + c_pos;
         live[ct] = c_pos < pos_per_wave && qrow[ct] < n_b;
         const int lim = causal ? kv_len - n_b + qrow[ct] + 1 : kv_len;
-        limit[ct] = live[ct] ? min(max(lim, 0), kv_len) : 0;
+        limit[ct] = live[ct] ? min(max(lim, 0), kv_cap) : 0;
         const uint16_t *qrow_p =
             q + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim + h * 8;
 #pragma unroll
@@ -132,12 +143,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     // and must be uniform for the compiler too.  The workgroup walks [0, t_end);
     // a wave computes on [0, w_end) and masks from w_mask_from on.
     const int rows_wg = min(kPrefillWaves * pos_per_wave, n_b - q0);          // >= 1 by construction
-    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_wg : kv_len, 0), kv_len);
+    const int t_first = blk_begin * kBlock;                                   // the walk starts here
+    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_wg : kv_len, 0), kv_cap);
     const int rows_w = min(pos_per_wave, n_b - wq0);                          // <= 0: idle wave
     const int w_mask_from =
-        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + 1 : kv_len, 0), kv_len) : 0;
-    const int w_end =
-        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + rows_w : kv_len, 0), kv_len) : 0;
+        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + 1 : kv_len, 0), kv_cap) : 0;
+    int w_end = rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + rows_w : kv_len, 0), kv_cap) : 0;
+    if (w_end <= t_first) w_end = 0;   // nothing of this part is visible to the wave's rows: idle
 
     const int n_blocks = (t_end + kBlock - 1) / kBlock;
     // Start value of the running maximum: far below any scaled score, far above a
@@ -167,12 +179,36 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const uint32_t one2 = E::pack2(1.f, 1.f);
     const u32x4 ones = {one2, one2, one2, one2};
 
-    // No kv token visible to any row of the tile: the output rows are zero.
-    // (Uniform over the workgroup, and before the first barrier.)
-    if (t_end == 0) {
+    // A plan that splits tiles: every part leaves (max, sum, unnormalised O) of its rows in
+    // slot row * n_splits + split of the workspace, laid out as the merge pass of the decode
+    // path reads it; a part that sees nothing leaves zeros and a maximum below any real one.
+    auto store_partial = [&](int ct, float m, float l) {
+        const long slot = (long)(q_begin + qrow[ct]) * n_splits + split;
+        if (slot >= max_slots) return;   // a slot beyond the workspace is never written
+        const long qh = (long)kvh * group + c_head[ct];
+        float *o = part_o + (slot * n_qo_heads + qh) * kHeadDim + 4 * h;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                *reinterpret_cast<f32x4 *>(o + dt * 32 + 8 * i) =
+                    f32x4{acc[ct][dt][4 * i], acc[ct][dt][4 * i + 1], acc[ct][dt][4 * i + 2], acc[ct][dt][4 * i + 3]};
+        if (h == 0) {
+            float *ml = part_ml + (slot * n_qo_heads + qh) * 2;
+            ml[0] = m;
+            ml[1] = l;
+        }
+    };
+    // No kv token of this part visible to any row of the tile: the output rows are zero
+    // (or the part is empty).  Uniform over the workgroup, and before the first barrier.
+    if (t_end <= t_first) {
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
             if (!live[ct]) continue;
+            if (n_splits > 1) {
+                store_partial(ct, m_run[ct], 0.f);
+                continue;
+            }
             uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
                           4 * h;
 #pragma unroll
@@ -361,35 +397,36 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 #pragma unroll
         for (int i = 0; i < kRowGroups; i++) zero[i] = z;
         store_rows(v_stage[3], zero);   // V(-1): multiplied by P(-1) = 0, must be finite
+        // the walk starts at block blk_begin, a multiple of four: block j still lives in stage j % 4
         if (kRowsSharePage) {
 #pragma unroll
-            for (int blk = 0; blk < 4; blk++) lookup_pages(blk, pg[blk]);
+            for (int blk = 0; blk < 4; blk++) lookup_pages(blk_begin + blk, pg[blk]);
 #pragma unroll
-            for (int blk = 0; blk < 4; blk++) prepare_rows(blk, pg[blk], desc[blk]);
+            for (int blk = 0; blk < 4; blk++) prepare_rows(blk_begin + blk, pg[blk], desc[blk]);
 #pragma unroll
             for (int blk = 0; blk < 3; blk++) load_direct(desc[blk].k, k_stage[blk]);
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) load_direct(desc[blk].v, v_stage[blk]);
-            lookup_pages(4, pg[0]);
+            lookup_pages(blk_begin + 4, pg[0]);
             DSKV_WAIT_VMEM(0);
         } else {
             u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
 #pragma unroll
-            for (int blk = 0; blk < 2; blk++) load_rows(blk, first_k[blk], first_v[blk]);
+            for (int blk = 0; blk < 2; blk++) load_rows(blk_begin + blk, first_k[blk], first_v[blk]);
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
                 store_rows(k_stage[blk], first_k[blk]);
                 store_rows(v_stage[blk], first_v[blk]);
             }
-            load_rows(2, even.k, even.v);
-            load_rows(3, odd.k, odd.v);
+            load_rows(blk_begin + 2, even.k, even.v);
+            load_rows(blk_begin + 3, odd.k, odd.v);
         }
     }
     __syncthreads();
     if (w_end > 0) {
         read_k_operands(k_stage[0]);
         scores(0);
-        if (kBlock > w_mask_from) mask_scores(0, 0);
+        if ((blk_begin + 1) * kBlock > w_mask_from) mask_scores(blk_begin, 0);
         block_max(0);
     }
     // V operand: token 16 ks + 8 hi + 4 h + (c >> 2) = row c >> 2 of region 4 ks + 2 hi + h;
@@ -512,7 +549,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
     };
-    for (int m = 0; m <= n_blocks; m += 4) {
+    for (int m = blk_begin; m <= n_blocks; m += 4) {
         iteration(m, 0, even);
         iteration(m + 1, 1, odd);
         iteration(m + 2, 2, even);
@@ -530,6 +567,10 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             l = l_run[ct] + l_other;
         }
         if (!live[ct]) continue;
+        if (n_splits > 1) {
+            store_partial(ct, m_run[ct], l);
+            continue;
+        }
         const float inv = l > 0.f ? 1.f / l : 0.f;
         uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
                       4 * h;
@@ -619,70 +660,132 @@ static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads)
 
 }  // namespace dskv
 
+namespace dskv {
+
+constexpr int kMaxPrefillSplits = 8;         // parts a tile's K/V range is cut into at most
+// a part holds at least this many tokens: with 256, a 512-token chunk without prior context
+// took 37 us in two parts instead of 29 us whole; with 1024, chunks over 1-2 k tokens of prior
+// context lost a fifth of what the parts buy
+constexpr int kMinSplitTokens = 512;
+constexpr int kMaxSplitTarget = 1024;        // workgroups a split plan aims at, at most
+constexpr int32_t kWholeRange = 0x7fffffff;  // blk_end of a tile that is not split
+
+static int compute_units()
+{
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    (void)hipGetLastError();
+    return cus;
+}
+
+}  // namespace dskv
+
 extern "C" int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz)
 {
+    using namespace dskv;
     if (batch < 0 || nnz < 0) return 0;
-    return 2 * ((int64_t)batch + nnz);
+    // entries: one per tile, or per part of a tile when the plan splits (then there are few
+    // tiles: at most 2 * kMaxSplitTarget parts); then two words per query row
+    return kTileWords * ((int64_t)batch + nnz + 2 * kMaxSplitTarget) + 2 * nnz;
 }
 
 extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
                                  int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads,
-                                 int32_t *tile_info_host, int64_t capacity_words,
-                                 int32_t *n_tiles_out)
+                                 int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
+                                 int64_t capacity_words, int32_t *n_tiles_out,
+                                 int32_t *n_splits_out, int64_t *plan_words_out,
+                                 int64_t *workspace_bytes_out)
 {
     using namespace dskv;
-    DSKV_REQUIRE(batch >= 0 && n_tiles_out, "prefill_plan: bad arguments");
+    DSKV_REQUIRE(batch >= 0 && n_tiles_out && n_splits_out && plan_words_out && workspace_bytes_out,
+                 "prefill_plan: bad arguments");
     DSKV_REQUIRE(n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0,
                  "prefill_plan: n_qo_heads %d not a multiple of n_kv_heads %d", n_qo_heads,
                  n_kv_heads);
     *n_tiles_out = 0;
+    *n_splits_out = 1;
+    *plan_words_out = 0;
+    *workspace_bytes_out = 0;
     if (batch == 0) return 0;
-    DSKV_REQUIRE(qo_indptr_host && tile_info_host, "prefill_plan: null pointer argument");
+    DSKV_REQUIRE(qo_indptr_host && plan_host, "prefill_plan: null pointer argument");
     const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads);
-    int64_t n = 0;
-    // later query tiles of a request see more keys: emit them first
+    // later query tiles of a request see more keys: they come first within a request
+    struct Tile { int32_t b, row; int64_t keys; };
+    std::vector<Tile> tiles;
+    int64_t nnz = 0;
     for (int b = 0; b < batch; b++) {
         const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
         DSKV_REQUIRE(n_b >= 0, "prefill_plan: qo_indptr not monotone at %d", b);
-        const int64_t tiles = (n_b + rows - 1) / rows;
-        if ((n + tiles) * 2 > capacity_words) {
-            set_error("prefill_plan: tile list needs more than %lld words", (long long)capacity_words);
-            return DSKV_E_NOMEM;
-        }
-        for (int64_t i = tiles - 1; i >= 0; i--) {
-            tile_info_host[2 * n] = b;
-            tile_info_host[2 * n + 1] = (int32_t)(i * rows);
-            n++;
+        nnz += n_b;
+        for (int64_t i = (n_b + rows - 1) / rows - 1; i >= 0; i--) {
+            const int64_t last_row = std::min<int64_t>(i * rows + rows, n_b) - 1;
+            const int64_t keys = kv_len_host ? std::max<int64_t>((int64_t)kv_len_host[b] - n_b + last_row + 1, 0) : 0;
+            tiles.push_back({b, (int32_t)(i * rows), keys});
         }
     }
-    DSKV_REQUIRE(n < (int64_t(1) << 31), "prefill_plan: too many tiles");
-    *n_tiles_out = (int32_t)n;
-    if (kv_len_host && n > 1) {
-        // Workgroups are dispatched in tile order and a tile's time grows with the keys its
-        // last row sees: longest first, so the short ones fill the end of the launch
-        // (request order left a fifth of the wave slots idle on mixed lengths).
-        struct Tile { int32_t b, row; int64_t keys; };
-        std::vector<Tile> order((size_t)n);
-        for (int64_t i = 0; i < n; i++) {
-            const int32_t b = tile_info_host[2 * i], row = tile_info_host[2 * i + 1];
-            const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
-            const int64_t last_row = std::min<int64_t>(row + rows, n_b) - 1;
-            order[(size_t)i] = {b, row, std::max<int64_t>((int64_t)kv_len_host[b] - n_b + last_row + 1, 0)};
-        }
-        std::stable_sort(order.begin(), order.end(),
+    DSKV_REQUIRE(tiles.size() < (size_t(1) << 26) && nnz < (int64_t(1) << 31), "prefill_plan: too many tiles");
+    // Workgroups are dispatched in plan order and a tile's time grows with the keys its
+    // last row sees: longest first, so the short ones fill the end of the launch
+    // (request order left a fifth of the wave slots idle on mixed lengths).
+    if (kv_len_host && tiles.size() > 1)
+        std::stable_sort(tiles.begin(), tiles.end(),
                          [](const Tile &x, const Tile &y) { return x.keys > y.keys; });
-        for (int64_t i = 0; i < n; i++) {
-            tile_info_host[2 * i] = order[(size_t)i].b;
-            tile_info_host[2 * i + 1] = order[(size_t)i].row;
+    // Few tiles (a chunk of a few hundred tokens, as the reference's scheduler hands out:
+    // one 512-token chunk of an 8-kv-head model is 64 workgroups) leave most of the chip
+    // idle: then every tile's K/V range is cut into parts that run as workgroups of their
+    // own and leave partials, merged by a second pass - the decode path's way of keeping
+    // all compute units busy.  Needs the kv lengths and the 16-bit kernel's head dim.
+    int splits = 1;
+    if (kv_len_host && head_dim == kHeadDim && target_workgroups >= 0 && !tiles.empty()) {
+        const int64_t target =
+            target_workgroups > 0 ? std::min<int64_t>(target_workgroups, kMaxSplitTarget) : compute_units();
+        const int64_t wgs = (int64_t)tiles.size() * n_kv_heads;
+        if (wgs * 2 <= target) {
+            splits = (int)std::min<int64_t>(kMaxPrefillSplits, target / wgs);
+            splits = (int)std::min<int64_t>(splits, std::max<int64_t>(1, tiles.front().keys / kMinSplitTokens));
         }
     }
+    const int64_t n_entries = (int64_t)tiles.size() * splits;
+    const int64_t words = n_entries * kTileWords + (splits > 1 ? 2 * nnz : 0);
+    if (words > capacity_words) {
+        set_error("prefill_plan: plan needs %lld words, buffer has %lld", (long long)words,
+                  (long long)capacity_words);
+        return DSKV_E_NOMEM;
+    }
+    int32_t *p = plan_host;
+    for (const Tile &t : tiles) {
+        // parts of equal length, in units of four 32-token blocks (the kernel's loop is
+        // unrolled by four); a part that starts past the tile's last block is empty
+        const int64_t blocks = (t.keys + kBlock - 1) / kBlock;
+        const int64_t chunk = ((blocks + splits - 1) / splits + 3) / 4 * 4;
+        for (int s = 0; s < splits; s++) {
+            *p++ = t.b;
+            *p++ = t.row;
+            *p++ = splits > 1 ? (int32_t)std::min<int64_t>(s * chunk, (blocks + 3) / 4 * 4) : 0;
+            *p++ = splits > 1 && s + 1 < splits ? (int32_t)((s + 1) * chunk) : kWholeRange;
+            *p++ = s;
+        }
+    }
+    if (splits > 1)
+        for (int64_t r = 0; r < nnz; r++) {
+            *p++ = (int32_t)(r * splits);
+            *p++ = splits;
+        }
+    *n_tiles_out = (int32_t)n_entries;
+    *n_splits_out = splits;
+    *plan_words_out = words;
+    *workspace_bytes_out =
+        splits > 1 ? nnz * splits * (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float) : 0;
     return 0;
 }
 
 extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr,
                                  const void *pages_layer, const int32_t *kv_page_indices,
                                  const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
-                                 const int32_t *tile_info_dev, int32_t n_tiles, int32_t batch,
+                                 const int32_t *plan_dev, int32_t n_tiles, int32_t n_splits,
+                                 void *workspace, int64_t workspace_bytes, int32_t batch,
                                  int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
                                  int32_t head_dim, int32_t page_size, float sm_scale,
                                  int32_t causal, int32_t dtype, void *stream)
@@ -707,7 +810,21 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     const bool mfma = (dtype == DSKV_BF16 || dtype == DSKV_F16) && head_dim == kHeadDim &&
                       n_qo_heads / n_kv_heads <= kWaveCols && scale_log2 > 1e-6f && scale_log2 < 1e6f;
     if (mfma) {
-        DSKV_REQUIRE(tile_info_dev && n_tiles > 0, "prefill_attn: missing tile list");
+        DSKV_REQUIRE(plan_dev && n_tiles > 0, "prefill_attn: missing plan");
+        DSKV_REQUIRE(n_splits >= 1 && n_splits <= kMaxPrefillSplits && n_tiles % n_splits == 0,
+                     "prefill_attn: %d plan entries in %d parts", n_tiles, n_splits);
+        float *part_o = nullptr, *part_ml = nullptr;
+        int64_t max_slots = 0;
+        if (n_splits > 1) {
+            const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
+            DSKV_REQUIRE(workspace && workspace_bytes >= (int64_t)nnz * n_splits * slot_bytes &&
+                             (uintptr_t)workspace % 16 == 0,
+                         "prefill_attn: a plan in %d parts needs a 16-byte aligned workspace of %lld bytes, got %lld",
+                         n_splits, (long long)((int64_t)nnz * n_splits * slot_bytes), (long long)workspace_bytes);
+            max_slots = std::min<int64_t>(workspace_bytes / slot_bytes, 1 << 30);
+            part_o = reinterpret_cast<float *>(workspace);
+            part_ml = part_o + max_slots * n_qo_heads * (int64_t)head_dim;
+        }
         DSKV_REQUIRE(((uintptr_t)out | (uintptr_t)q | (uintptr_t)pages_layer) % 16 == 0,
                      "prefill_attn: out/q/pages must be 16-byte aligned");
         DSKV_REQUIRE(is_pow2(page_size),
@@ -719,8 +836,9 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
 #define DSKV_LAUNCH_PREFILL(DT, SHARE)                                                          \
     hipLaunchKernelGGL((prefill_attn_mfma_kernel<DT, SHARE>), grid, block, 0, s, (uint16_t *)out, \
                        (const uint16_t *)q, qo_indptr, (const char *)pages_layer,               \
-                       kv_page_indices, kv_page_indptr, kv_last_page_len, tile_info_dev,        \
-                       n_qo_heads, n_kv_heads, shift, scale_log2, causal)
+                       kv_page_indices, kv_page_indptr, kv_last_page_len, plan_dev,             \
+                       n_qo_heads, n_kv_heads, shift, scale_log2, causal, n_splits, part_o,     \
+                       part_ml, (int)max_slots)
         if (dtype == DSKV_BF16) {
             if (page_size >= 4) DSKV_LAUNCH_PREFILL(DSKV_BF16, true);
             else DSKV_LAUNCH_PREFILL(DSKV_BF16, false);
@@ -730,6 +848,9 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
         }
 #undef DSKV_LAUNCH_PREFILL
         DSKV_LAUNCH_CHECK("prefill_attn_mfma_kernel");
+        if (n_splits > 1)   // the parts' partials become the output rows
+            return launch_partials_merge(out, part_o, part_ml, plan_dev + (int64_t)n_tiles * kTileWords,
+                                         (int)max_slots, nnz, n_qo_heads, head_dim, dtype, false, s);
     } else {
         dim3 grid((unsigned)nnz, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_GEN(DT)                                                                      \

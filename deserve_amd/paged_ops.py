@@ -324,10 +324,15 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
                       qo_indptr_host: Optional[torch.Tensor] = None,
                       paged_kv_indptr_host: Optional[torch.Tensor] = None,
                       paged_kv_last_page_len_host: Optional[torch.Tensor] = None,
-                      paged_kv_indices_host: Optional[torch.Tensor] = None, **_ignored) -> None:
+                      paged_kv_indices_host: Optional[torch.Tensor] = None,
+                      target_workgroups: int = 0, **_ignored) -> None:
         """The *_host arguments are host copies of the index tensors (the planner and the
         checks of the block tables run on the host; without them the device tensors are read
-        back, which synchronises)."""
+        back, which synchronises).
+        target_workgroups: a batch of few query tiles (a chunk of a few hundred tokens) is
+        planned in several parts per tile, merged by a second pass, so that the launch has
+        about this many workgroups (0: one per compute unit; negative: never split); the parts'
+        partials go to the workspace buffer."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
@@ -343,19 +348,23 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         self._check_block_tables(h_kv, paged_kv_indices, paged_kv_indices_host, h_last32)
         L = _lib.lib()
         cap = L.dskv_prefill_plan_bound(batch, nnz)
-        block = staging.take(max(cap, 2))
+        block = staging.take(max(cap, 4))
         tiles = block.tensor
-        n_tiles = ctypes.c_int32()
+        n_tiles, n_splits = ctypes.c_int32(), ctypes.c_int32()
+        words, ws = ctypes.c_int64(), ctypes.c_int64()
         # kv lengths order the tiles longest first
         h_indptr = h_kv.to(torch.int64)
         h_last = h_last32.to(torch.int64)
         n_pages = h_indptr[1:] - h_indptr[:-1]
         kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
         rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,
-                                 tiles.data_ptr(), cap, ctypes.byref(n_tiles))
+                                 head_dim, target_workgroups, tiles.data_ptr(), cap, ctypes.byref(n_tiles),
+                                 ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
         _lib.check(rc, "prefill begin_forward")
-        self._batch, self._nnz, self._n_tiles = batch, nnz, n_tiles.value
-        self._tiles = staging.to_device(block, max(2 * n_tiles.value, 2), paged_kv_indices.device)
+        if ws.value > self._workspace.numel() * self._workspace.element_size():
+            raise RuntimeError(f"prefill workspace too small: need {ws.value} bytes")
+        self._batch, self._nnz, self._n_tiles, self._n_splits = batch, nnz, n_tiles.value, n_splits.value
+        self._tiles = staging.to_device(block, max(int(words.value), 4), paged_kv_indices.device)
         self._planned = True
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor, causal: bool = True,
@@ -371,7 +380,9 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         rc = _lib.lib().dskv_prefill_attn(
             out.data_ptr(), q.data_ptr(), self._qo_indptr.data_ptr(), paged_kv_data.data_ptr(),
             self._indices.data_ptr(), self._indptr.data_ptr(), self._last.data_ptr(),
-            self._tiles.data_ptr(), self._n_tiles, self._batch, self._nnz, self._hq, self._hkv,
-            self._d, self._p, scale, int(causal), _lib.dtype_code(q.dtype), _lib.current_stream())
+            self._tiles.data_ptr(), self._n_tiles, self._n_splits, self._workspace.data_ptr(),
+            self._workspace.numel() * self._workspace.element_size(), self._batch, self._nnz, self._hq,
+            self._hkv, self._d, self._p, scale, int(causal), _lib.dtype_code(q.dtype),
+            _lib.current_stream())
         _lib.check(rc, "prefill forward")
         return out

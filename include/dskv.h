@@ -192,24 +192,39 @@ int dskv_decode_rope_append_attn(void *out, const void *q, const void *k_new, co
  * (model/layer/attention.py:188-192, execution/exec.py:227-236).
  * q, out: (nnz, n_qo_heads, head_dim); qo_indptr (batch+1) device int32.
  * Query i of the n_b queries of request b sees kv positions
- * j <= kv_len_b - n_b + i.  tile_info_dev: (n_tiles, 2) int32 pairs
- * (request, first query row of the tile within the request) built by
- * dskv_prefill_plan from the host copy of qo_indptr (needs at most
- * dskv_prefill_plan_bound(batch, nnz) words); unused (may be NULL) for fp32.
- * kv_len_host (batch host int32, may be NULL): the requests' kv lengths; with
- * them the tiles are ordered longest first, which balances a launch over
- * requests of mixed lengths (the result does not depend on the order).
+ * j <= kv_len_b - n_b + i.
+ *
+ * dskv_prefill_plan (host; replaces the planning half of begin_forward,
+ * execution/exec.py:227-236) cuts the requests' query rows into tiles, one
+ * workgroup per tile and kv head, and writes the plan - at most
+ * dskv_prefill_plan_bound(batch, nnz) words - that dskv_prefill_attn reads from
+ * device memory (plan_dev: the first *plan_words_out words, uploaded by the caller;
+ * unused, may be NULL, for fp32).
+ * kv_len_host (batch host int32, may be NULL): the requests' kv lengths.  With
+ * them the tiles are ordered longest first, which balances a launch over requests
+ * of mixed lengths, and a batch of few tiles (the 512-token chunks of the
+ * reference's scheduler, engine/pipeline/scheduler.py:74,85: 64 workgroups for an
+ * 8-kv-head model) is planned in *n_splits_out > 1 parts per tile: every part walks
+ * a slice of the tile's K/V as a workgroup of its own and leaves partials in the
+ * workspace (*workspace_bytes_out bytes, 16-byte aligned), which dskv_prefill_attn
+ * merges in a second pass.  target_workgroups: workgroups such a plan aims at
+ * (0: one per compute unit; negative: never split).  The result does not depend
+ * on the order of the tiles, and on the parts only in the last bits.
+ * n_tiles: *n_tiles_out (plan entries: tiles times parts).
  */
 int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz);
 int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host, int32_t batch,
-                      int32_t n_qo_heads, int32_t n_kv_heads, int32_t *tile_info_host,
-                      int64_t capacity_words, int32_t *n_tiles_out);
+                      int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                      int32_t target_workgroups, int32_t *plan_host, int64_t capacity_words,
+                      int32_t *n_tiles_out, int32_t *n_splits_out, int64_t *plan_words_out,
+                      int64_t *workspace_bytes_out);
 int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const void *pages_layer,
                       const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
-                      const int32_t *kv_last_page_len, const int32_t *tile_info_dev,
-                      int32_t n_tiles, int32_t batch, int32_t nnz, int32_t n_qo_heads,
-                      int32_t n_kv_heads, int32_t head_dim, int32_t page_size, float sm_scale,
-                      int32_t causal, int32_t dtype, void *stream);
+                      const int32_t *kv_last_page_len, const int32_t *plan_dev, int32_t n_tiles,
+                      int32_t n_splits, void *workspace, int64_t workspace_bytes, int32_t batch,
+                      int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                      int32_t page_size, float sm_scale, int32_t causal, int32_t dtype,
+                      void *stream);
 
 /*
  * Rotary embedding, adjacent-pair convention.  Replaces the call site

@@ -159,15 +159,31 @@ def test_decode_plan_rejects_bad_metadata_and_small_buffers():
     assert lib.dskv_decode_plan(indptr.ctypes.data, last.ctypes.data, *small) == -2
 
 
+def _prefill_plan(lib, qo, kv_len, hq, hkv, target=0, head_dim=128, cap=None):
+    """Runs dskv_prefill_plan; returns (rc, entries (n, 5), n_splits, row parts or None, workspace bytes)."""
+    batch, nnz = len(qo) - 1, int(qo[-1])
+    cap = lib.dskv_prefill_plan_bound(batch, nnz) if cap is None else cap
+    plan = np.zeros(max(cap, 8), np.int32)
+    n, splits = ctypes.c_int32(), ctypes.c_int32()
+    words, ws = ctypes.c_int64(), ctypes.c_int64()
+    rc = lib.dskv_prefill_plan(qo.ctypes.data, None if kv_len is None else kv_len.ctypes.data, batch, hq, hkv,
+                               head_dim, target, plan.ctypes.data, cap, ctypes.byref(n), ctypes.byref(splits),
+                               ctypes.byref(words), ctypes.byref(ws))
+    if rc:
+        return rc, None, None, None, None
+    entries = plan[: 5 * n.value].reshape(-1, 5)
+    parts = plan[5 * n.value: words.value].reshape(-1, 2) if splits.value > 1 else None
+    assert words.value == 5 * n.value + (0 if parts is None else 2 * nnz)
+    return rc, entries, splits.value, parts, ws.value
+
+
 def test_prefill_plan_tiles_cover_all_query_rows():
     lib = _lib.lib()
     qo = np.array([0, 512, 512, 519, 520], np.int32)
     for hq, hkv in [(32, 8), (64, 8), (8, 8), (32, 1)]:
-        cap = lib.dskv_prefill_plan_bound(4, 520)
-        tiles = np.zeros(cap, np.int32)
-        n = ctypes.c_int32()
-        assert lib.dskv_prefill_plan(qo.ctypes.data, None, 4, hq, hkv, tiles.ctypes.data, cap, ctypes.byref(n)) == 0
-        t = tiles[: 2 * n.value].reshape(-1, 2)
+        rc, t, splits, parts, ws = _prefill_plan(lib, qo, None, hq, hkv)
+        assert rc == 0 and splits == 1 and parts is None and ws == 0
+        assert (t[:, 2] == 0).all() and (t[:, 3] == 0x7fffffff).all() and (t[:, 4] == 0).all()
         group = hq // hkv
         rows = None
         for b in range(4):
@@ -181,8 +197,7 @@ def test_prefill_plan_tiles_cover_all_query_rows():
                 # a tile is a whole number of waves, each 32 // group query rows
                 assert rows % max(32 // group, 1) == 0 if group <= 32 else rows == 1
             assert starts == list(range(0, nb, rows))
-    n = ctypes.c_int32()
-    assert lib.dskv_prefill_plan(qo.ctypes.data, None, 4, 32, 8, tiles.ctypes.data, 4, ctypes.byref(n)) == -2
+    assert _prefill_plan(lib, qo, None, 32, 8, cap=4)[0] == -2
 
 
 def test_prefill_plan_with_kv_lengths_orders_tiles_longest_first():
@@ -190,17 +205,51 @@ def test_prefill_plan_with_kv_lengths_orders_tiles_longest_first():
     lib = _lib.lib()
     qo = np.array([0, 512, 512, 519, 520, 1000], np.int32)
     kv_len = np.array([600, 0, 4000, 1, 480], np.int32)
-    cap = lib.dskv_prefill_plan_bound(5, 1000)
-    plain, ordered = np.zeros(cap, np.int32), np.zeros(cap, np.int32)
-    n0, n1 = ctypes.c_int32(), ctypes.c_int32()
-    assert lib.dskv_prefill_plan(qo.ctypes.data, None, 5, 32, 8, plain.ctypes.data, cap, ctypes.byref(n0)) == 0
-    assert lib.dskv_prefill_plan(qo.ctypes.data, kv_len.ctypes.data, 5, 32, 8, ordered.ctypes.data, cap,
-                                 ctypes.byref(n1)) == 0
-    assert n0.value == n1.value
-    a = plain[: 2 * n0.value].reshape(-1, 2)
-    b = ordered[: 2 * n1.value].reshape(-1, 2)
+    _, a, s0, _, _ = _prefill_plan(lib, qo, None, 32, 8)
+    _, b, s1, _, _ = _prefill_plan(lib, qo, kv_len, 32, 8, target=-1)
+    assert s0 == s1 == 1 and len(a) == len(b)
     assert sorted(map(tuple, a.tolist())) == sorted(map(tuple, b.tolist()))
     rows = 64                                             # 8 waves x 32 // 4 query rows
     n_b = np.diff(qo)
-    keys = [kv_len[r] - n_b[r] + min(s + rows, n_b[r]) for r, s in b]
+    keys = [kv_len[r] - n_b[r] + min(s + rows, n_b[r]) for r, s in b[:, :2]]
     assert keys == sorted(keys, reverse=True) and keys[0] == 4000
+
+
+def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
+    """One 512-token chunk over 4096 prior tokens is 8 tiles x 8 kv heads = 64 workgroups: for
+    256 it is planned in 4 parts per tile.  The parts of a tile are consecutive block ranges
+    that start at multiples of four blocks and cover [0, blocks of the tile); every query row
+    gets its run of slots; a full batch, a plan without lengths or with another head dim,
+    and target < 0 are not split."""
+    lib = _lib.lib()
+    qo = np.array([0, 512], np.int32)
+    kv_len = np.array([4096 + 512], np.int32)
+    rc, t, splits, parts, ws = _prefill_plan(lib, qo, kv_len, 32, 8, target=256)
+    assert rc == 0 and splits == 4 and len(t) == 8 * 4
+    assert ws == 512 * 4 * 32 * (128 + 2) * 4
+    assert parts.tolist() == [[r * 4, 4] for r in range(512)]
+    for row in range(0, 512, 64):
+        mine = t[t[:, 1] == row]
+        assert mine[:, 0].tolist() == [0] * 4 and mine[:, 4].tolist() == [0, 1, 2, 3]
+        blocks = -(-(4096 + row + 64) // 32)              # keys the tile's last row sees, in blocks
+        begin, end = mine[:, 2].tolist(), mine[:, 3].tolist()
+        assert begin[0] == 0 and all(x % 4 == 0 for x in begin) and end[-1] == 0x7fffffff
+        assert end[:-1] == begin[1:] and begin[-1] < blocks
+    # the longest tile first
+    assert t[0, 1] == 448
+    # short keys limit the parts: a part holds at least 512 tokens
+    assert _prefill_plan(lib, qo, np.array([700], np.int32), 32, 8, target=256)[2] == 1
+    assert _prefill_plan(lib, qo, np.array([1100], np.int32), 32, 8, target=256)[2] == 2
+    assert _prefill_plan(lib, qo, np.array([2100], np.int32), 32, 8, target=256)[2] == 4
+    # not split: no lengths, another head dim, target < 0, enough tiles already
+    assert _prefill_plan(lib, qo, None, 32, 8, target=256)[2] == 1
+    assert _prefill_plan(lib, qo, kv_len, 32, 8, target=256, head_dim=64)[2] == 1
+    assert _prefill_plan(lib, qo, kv_len, 32, 8, target=-1)[2] == 1
+    big = np.array([0, 2048], np.int32)
+    assert _prefill_plan(lib, big, np.array([4096], np.int32), 32, 8, target=256)[2] == 1
+    # a part past a tile's last block is empty: begin is clamped to the tile's blocks (rounded up to four)
+    qo2 = np.array([0, 64, 128], np.int32)
+    rc, t, splits, parts, ws = _prefill_plan(lib, qo2, np.array([4096, 100], np.int32), 32, 8, target=256)
+    assert splits == 8
+    short = t[t[:, 0] == 1]
+    assert short[:, 2].tolist() == [0] + [4] * 7

@@ -251,6 +251,9 @@ PREFILL_CASES = [
     ("long_tile", [900], [300], 16, 32, 8, 128, "bf16"),
     ("no_kv", [0, 40], [2, 8], 16, 32, 8, 128, "bf16"),
     ("more_queries_than_kv", [5, 33, 64], [9, 40, 64], 16, 32, 8, 128, "bf16"),
+    # few tiles over long keys: planned in 4 and 8 parts per tile, most parts of the short requests empty
+    ("split_parts", [5000, 1100, 40], [200, 130, 40], 16, 32, 8, 128, "bf16"),
+    ("split_parts_f16_page8_group8", [3000, 2049], [65, 1], 8, 64, 8, 128, "f16"),
 ]
 
 
@@ -261,18 +264,31 @@ def test_prefill_attention_matches_oracle(case):
     name, kv, qo, P, Hq, Hkv, D, dtype = case
     _announce("prefill", *case)
     sc = make_scenario(41, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=D, dtype=dtype)
-    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
-    w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
-                    _dev_i32(sc.kv_last_page_lens), Hq, Hkv, D, P)
-    for causal in (True, False):
-        out = w.forward(to_torch(sc.q, dtype), to_torch(sc.pages, dtype), causal=causal)
-        torch.cuda.synchronize()
-        got = out.float().cpu().numpy()
-        want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
-                                     sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
-        assert np.isfinite(got).all()
-        assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (name, causal)
-    w.end_forward()
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
+    want = {causal: c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
+                                          sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
+            for causal in (True, False)}
+    # the plan as it comes (these few tiles are cut into parts wherever the keys allow), in
+    # as many parts as possible, and whole tiles
+    parts_seen = set()
+    for target in (0, 1024, -1):
+        w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                        _dev_i32(sc.kv_last_page_lens), Hq, Hkv, D, P, target_workgroups=target)
+        parts_seen.add(w._n_splits)
+        for causal in (True, False):
+            out = w.forward(to_torch(sc.q, dtype), to_torch(sc.pages, dtype), causal=causal)
+            torch.cuda.synchronize()
+            got = out.float().cpu().numpy()
+            assert np.isfinite(got).all()
+            assert max_rel_err_per_request(got, want[causal]) <= ATTN_TOL[dtype], (name, causal, target, w._n_splits)
+        w.end_forward()
+    assert 1 in parts_seen
+    if name == "ragged_prior":
+        assert max(parts_seen) > 1, parts_seen
+    if name == "split_parts":
+        assert parts_seen == {1, 4, 8}, parts_seen
+    if name == "split_parts_f16_page8_group8":
+        assert parts_seen == {1, 5}, parts_seen
 
 
 def test_prefill_attention_random_shapes():
@@ -281,7 +297,7 @@ def test_prefill_attention_random_shapes():
     from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
 
     rng = np.random.default_rng(77)
-    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
     done = 0
     while done < 40:
         P = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
@@ -430,7 +446,7 @@ def test_prefill_with_one_query_equals_decode():
     _announce("prefill n=1 vs decode")
     sc = make_scenario(42, kv_lens=[700, 33, 16], qo_lens=[1, 1, 1], dtype="bf16")
     dec, _ = _run_decode(sc, 1)
-    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device="cuda"))
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
     w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                     _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P)
     pre = w.forward(to_torch(sc.q, "bf16"), to_torch(sc.pages, "bf16")).float().cpu().numpy()
