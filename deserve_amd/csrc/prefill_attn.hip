@@ -23,6 +23,11 @@
 //
 // Workgroup ids are laid out head-fastest: consecutive ids go to different XCDs,
 // so (with 8 kv heads) all query tiles of one kv head share one XCD's L2.
+//
+// A batch of few tiles (one 512-token chunk: 8 tiles x 8 kv heads) would leave most
+// of the chip idle.  The plan then cuts every tile's K/V range into parts; a part is
+// a workgroup of its own that leaves (maximum, sum, unnormalised O) of its rows in a
+// workspace, and the merge pass of the decode path turns the parts into the output.
 #include "kv_tile.h"
 
 #include <vector>
