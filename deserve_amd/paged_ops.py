@@ -357,12 +357,14 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         h_last = h_last32.to(torch.int64)
         n_pages = h_indptr[1:] - h_indptr[:-1]
         kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
-        rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,
-                                 head_dim, target_workgroups, tiles.data_ptr(), cap, ctypes.byref(n_tiles),
-                                 ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
-        _lib.check(rc, "prefill begin_forward")
-        if ws.value > self._workspace.numel() * self._workspace.element_size():
-            raise RuntimeError(f"prefill workspace too small: need {ws.value} bytes")
+        for target in (target_workgroups, -1):
+            rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,
+                                     head_dim, target, tiles.data_ptr(), cap, ctypes.byref(n_tiles),
+                                     ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
+            _lib.check(rc, "prefill begin_forward")
+            # a workspace too small for the parts' partials: whole tiles need none
+            if ws.value <= self._workspace.numel() * self._workspace.element_size():
+                break
         self._batch, self._nnz, self._n_tiles, self._n_splits = batch, nnz, n_tiles.value, n_splits.value
         self._tiles = staging.to_device(block, max(int(words.value), 4), paged_kv_indices.device)
         self._planned = True

@@ -99,3 +99,19 @@ def test_graph_key_holds_the_item_count_only_for_the_kernel_launched_per_item():
     assert key(4, 4, 5, q, False) == key(4, 4, 5, q, False)
     assert key(4, 4, 5, q, False) != key(4, 4, 5, q, True)
     assert key(4, 4, 5, q, True) != key(3, 4, 5, q, True) and key(4, 4, 5, q, True) != key(4, 8, 5, q, True)
+
+
+@pytest.mark.gpu
+def test_prefill_plan_falls_back_to_whole_tiles_when_the_workspace_cannot_hold_the_parts():
+    """One 512-token chunk over 4096 tokens is planned in parts that need 34 MB of partials;
+    with a 1 MiB workspace the wrapper plans whole tiles instead (no workspace needed)."""
+    dev = torch.device("cuda")
+    qo, kv_indptr = _i32([0, 512]).to(dev), _i32([0, 288]).to(dev)
+    ids, last = torch.arange(288, dtype=torch.int32, device=dev), _i32([16]).to(dev)
+    shape = dict(num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16, target_workgroups=256)
+    small = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device=dev))
+    big = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+    for w in (small, big):
+        w.begin_forward(qo, kv_indptr, ids, last, **shape)
+    assert (small._n_splits, small._n_tiles) == (1, 8)
+    assert (big._n_splits, big._n_tiles) == (4, 32)
