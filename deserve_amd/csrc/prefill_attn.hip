@@ -628,24 +628,51 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
         acc[i] = 0.f;
     }
     float m_run = kNegBig, l_run = 0.f;
-    for (int t = 0; t < limit; t++) {
-        const long page = kv_indices[page_begin + t / page_size];
-        const long base = page * 2 * half + (long)(t % page_size) * tok_row + (long)kvh * head_dim;
-        float dot = 0.f;
+    // kGroup tokens at a time: page ids, K rows and V rows of the group are all requested
+    // before the first is used (token by token, every token waited for memory twice)
+    constexpr int kGroup = 8;
+    for (int t0 = 0; t0 < limit; t0 += kGroup) {
+        long base[kGroup];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int d = lane + 64 * i;
-            if (d < head_dim) dot += qv[i] * L::get(pages, base + d);
+        for (int j = 0; j < kGroup; j++) {
+            const int t = min(t0 + j, limit - 1);   // past the limit: the last token again, weight zero
+            const long page = kv_indices[page_begin + t / page_size];
+            base[j] = page * 2 * half + (long)(t % page_size) * tok_row + (long)kvh * head_dim;
         }
-        const float x = wave_sum(dot) * scale_log2;
-        const float m_new = fmaxf(m_run, x);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        const float p = __builtin_amdgcn_exp2f(x - m_new);
-        l_run = l_run * alpha + p;
+        float kx[kGroup][4], vx[kGroup][4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int d = lane + 64 * i;
-            if (d < head_dim) acc[i] = acc[i] * alpha + p * L::get(pages, base + half + d);
+        for (int j = 0; j < kGroup; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int d = lane + 64 * i;
+                kx[j][i] = d < head_dim ? L::get(pages, base[j] + d) : 0.f;
+            }
+#pragma unroll
+        for (int j = 0; j < kGroup; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int d = lane + 64 * i;
+                vx[j][i] = d < head_dim ? L::get(pages, base[j] + half + d) : 0.f;
+            }
+        float x[kGroup], m_new = m_run;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) dot += qv[i] * kx[j][i];
+            x[j] = t0 + j < limit ? wave_sum(dot) * scale_log2 : kNegBig;
+            m_new = fmaxf(m_new, x[j]);
+        }
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] *= alpha;
+#pragma unroll
+        for (int j = 0; j < kGroup; j++) {
+            const float p = x[j] > kNegBig ? __builtin_amdgcn_exp2f(x[j] - m_new) : 0.f;
+            l_run += p;
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] += p * vx[j][i];
         }
         m_run = m_new;
     }
