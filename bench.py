@@ -62,6 +62,10 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--section", choices=["swap", "fragmented", "prefill"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
+    ap.add_argument("--prefill-config4-only", action="store_true",
+                    help="with --section prefill: only configuration 4's launches on its own data "
+                         "(20 appends, 20 attention launches), for profiler runs whose per-kernel "
+                         "averages must not mix in the zero-data and one-chunk measurements")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -321,7 +325,7 @@ def swap_section(seed: int):
             "streams_run_beside_compute": independent}
 
 
-def prefill_section(seed: int):
+def prefill_section(seed: int, extras: bool = True):
     """Baseline configuration 4 (Llama-3-8B stage): 16 sequences each append a 512-token chunk
     at a start offset U[0,15] inside a partially filled page and attend over a prior context
     U[0,8192].  Timed per layer on the launch stream: the chunk append and the paged prefill
@@ -380,6 +384,18 @@ def prefill_section(seed: int):
 
     append_us = median_us(append)
     attn_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
+    result = {"workload": "BASELINE.json configs[3]: bf16, GQA 32q/8kv, page 16, 16 sequences x 512-token "
+                          "chunk appended at offsets U[0,15], attention over prior U[0,8192]; per layer",
+              "chunk_tokens": B * n, "kv_tokens": int((prior + n).sum()),
+              "append_us_per_layer": round(append_us, 1),
+              "append_GBps": round(2 * B * n * 2 * Hkv * D * 2 / append_us / 1e3, 1),
+              "attention_us_per_layer": round(attn_us, 1),
+              "attention_TFLOPs": round(flops / attn_us / 1e6, 1),
+              "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
+              "flops_per_layer": flops}
+    if not extras:
+        w.end_forward()
+        return result
     # The same launches over all-zero q, K and V: instruction for instruction the same work,
     # only the operand bits differ.  The matrix pipeline then draws less power and the chip
     # keeps its clock; the gap to the figure above is what the power limit costs on
@@ -388,8 +404,6 @@ def prefill_section(seed: int):
     pool.pages.zero_()
     attn_zero_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
     w.end_forward()
-    append_bytes = 2 * B * n * 2 * Hkv * D * 2
-
     # One 512-token chunk over 4096 prior tokens: the step budget of the reference's scheduler
     # (engine/pipeline/scheduler.py:74,85).  8 query tiles x 8 kv heads are 64 workgroups, so
     # the plan cuts every tile's K/V range into parts (merged by a second pass); timed with
@@ -427,18 +441,10 @@ def prefill_section(seed: int):
     one_flops = 4 * Hq * D * (n * one_prior + n * (n + 1) // 2)
     for v in one_chunk.values():
         v["TFLOPs"] = round(one_flops / v["us_per_layer"] / 1e6, 1)
-    return {"workload": "BASELINE.json configs[3]: bf16, GQA 32q/8kv, page 16, 16 sequences x 512-token "
-                        "chunk appended at offsets U[0,15], attention over prior U[0,8192]; per layer",
-            "chunk_tokens": B * n, "kv_tokens": int((prior + n).sum()),
-            "append_us_per_layer": round(append_us, 1),
-            "append_GBps": round(append_bytes / append_us / 1e3, 1),
-            "attention_us_per_layer": round(attn_us, 1),
-            "attention_TFLOPs": round(flops / attn_us / 1e6, 1),
-            "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
-            "attention_us_per_layer_zero_data": round(attn_zero_us, 1),
-            "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
-            "flops_per_layer": flops,
-            "one_512_token_chunk_over_4096": one_chunk}
+    result.update({"attention_us_per_layer_zero_data": round(attn_zero_us, 1),
+                   "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
+                   "one_512_token_chunk_over_4096": one_chunk})
+    return result
 
 
 def fragmented_section(seed: int):
@@ -572,8 +578,10 @@ def main() -> int:
     if a.section is not None:
         import torch
         torch.cuda.set_device(0)
-        print(json.dumps({"swap": swap_section, "fragmented": fragmented_section,
-                          "prefill": prefill_section}[a.section](a.seed)))
+        if a.section == "prefill":
+            print(json.dumps(prefill_section(a.seed, extras=not a.prefill_config4_only)))
+        else:
+            print(json.dumps({"swap": swap_section, "fragmented": fragmented_section}[a.section](a.seed)))
         return 0
     if a.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {a.gpus} is not supported in this build "
