@@ -120,16 +120,9 @@ class BatchPrefill(BatchExec):
     def prepare(self) -> None:
         with torch.inference_mode():
             _, wrapper = get_wrappers(self.kvcaches[0].pool.main_device)
-            ctx = FlashPrefillCtx.init_paged_prefill_ctx(self.task_datas, self.kvcaches, wrapper)
-            wrapper.begin_forward(qo_indptr=ctx.indptr, paged_kv_indptr=ctx.kv_page_indptr,
-                                  paged_kv_indices=ctx.kv_page_indices,
-                                  paged_kv_last_page_len=ctx.kv_last_page_lens,
-                                  qo_indptr_host=ctx.host["indptr"],
-                                  paged_kv_indptr_host=ctx.host["kv_page_indptr"],
-                                  paged_kv_last_page_len_host=ctx.host["kv_last_page_lens"],
-                                  paged_kv_indices_host=ctx.host["kv_page_indices"],
-                                  **self._shape_kwargs())
-            self.prefill_ctx = ctx
+            # metadata and plan in one pinned block, one upload kernel
+            self.prefill_ctx = FlashPrefillCtx.init_and_plan(self.task_datas, self.kvcaches, wrapper,
+                                                             **self._shape_kwargs())
 
     def step(self, ignore_eos: bool) -> BatchResult:
         with torch.inference_mode():

@@ -217,3 +217,30 @@ class FlashPrefillCtx(FlashForwardCtx):
                                kvcaches: List[PagedKVCache[GpuPagePool]],
                                wrapper: BatchPrefillWithPagedKVCacheWrapper) -> "FlashPrefillCtx":
         return cls.init_paged_forward_ctx(task_datas, kvcaches, prefill_wrapper=wrapper)
+
+    @classmethod
+    def init_and_plan(cls, task_datas: List[TaskData], kvcaches: List[PagedKVCache[GpuPagePool]],
+                      wrapper: BatchPrefillWithPagedKVCacheWrapper, num_qo_heads: int, num_kv_heads: int,
+                      head_dim: int, page_size: int, target_workgroups: int = 0) -> "FlashPrefillCtx":
+        """init_paged_prefill_ctx + wrapper.begin_forward as ONE upload, as
+        FlashDecodeCtx.init_and_plan does for decode (what BatchPrefill.prepare does; the
+        reference: flash.py:46-64, exec.py:227-236)."""
+        pool = kvcaches[0].pool
+        meta = build_host_metadata(task_datas, kvcaches)
+        starts, total = metadata_layout(meta)
+        host = {f: torch.from_numpy(meta[f]) for f in _FIELDS}
+
+        def fill(view: torch.Tensor) -> None:
+            arr = view.numpy()
+            for f in _FIELDS:
+                arr[starts[f]: starts[f] + meta[f].shape[0]] = meta[f]
+
+        dev = wrapper.begin_forward_with_metadata(
+            total, fill, starts, host["indptr"], host["kv_page_indptr"], host["kv_last_page_lens"],
+            host["kv_page_indices"], num_qo_heads, num_kv_heads, head_dim, page_size, pool.main_device,
+            target_workgroups)
+        v = {f: dev[starts[f]: starts[f] + meta[f].shape[0]] for f in _FIELDS}
+        return cls(bsz=len(task_datas), seqlens=v["seqlens"], layer_id=0, page_pool=pool,
+                   offsets=v["offsets"], indptr=v["indptr"], kv_page_indices=v["kv_page_indices"],
+                   kv_page_indptr=v["kv_page_indptr"], kv_last_page_lens=v["kv_last_page_lens"],
+                   host=host, prefill_wrapper=wrapper)

@@ -337,37 +337,81 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
         h_qo = self._host(qo_indptr, qo_indptr_host)
+        h_kv = self._host(paged_kv_indptr, paged_kv_indptr_host)
+        h_last = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host)
+        cap, kv_len = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices, paged_kv_indices_host)
+        block = staging.take(max(cap, 4))
+        words = self._plan_into(block.tensor, cap, h_qo, kv_len, target_workgroups)
+        self._tiles = staging.to_device(block, max(words, 4), paged_kv_indices.device)
+        self._planned = True
+
+    def _check_and_bound(self, h_qo: torch.Tensor, h_kv: torch.Tensor, h_last: torch.Tensor,
+                         indices: torch.Tensor, indices_host: Optional[torch.Tensor]):
+        """Host-side checks of the index arrays; returns (words the plan may need, kv lengths)."""
         batch = h_qo.shape[0] - 1
-        nnz = int(h_qo[-1]) if batch > 0 else 0
         if batch > 0 and (int(h_qo[0]) != 0 or bool((h_qo[1:] < h_qo[:-1]).any())):
             raise ValueError("qo_indptr must start at 0 and not decrease")
-        h_kv = self._host(paged_kv_indptr, paged_kv_indptr_host)
         if h_kv.shape[0] != h_qo.shape[0]:
             raise ValueError("qo_indptr and paged_kv_indptr disagree about the batch")
-        h_last32 = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host)
-        self._check_block_tables(h_kv, paged_kv_indices, paged_kv_indices_host, h_last32)
-        L = _lib.lib()
-        cap = L.dskv_prefill_plan_bound(batch, nnz)
-        block = staging.take(max(cap, 4))
-        tiles = block.tensor
+        self._check_block_tables(h_kv, indices, indices_host, h_last)
+        nnz = int(h_qo[-1]) if batch > 0 else 0
+        h_indptr = h_kv.to(torch.int64)
+        n_pages = h_indptr[1:] - h_indptr[:-1]
+        kv_len = torch.where(n_pages > 0, (n_pages - 1) * self._p + h_last[:max(batch, 0)].to(torch.int64),
+                             n_pages).to(torch.int32)
+        return int(_lib.lib().dskv_prefill_plan_bound(batch, nnz)), kv_len
+
+    def _plan_into(self, plan: torch.Tensor, cap: int, h_qo: torch.Tensor, kv_len: torch.Tensor,
+                   target_workgroups: int) -> int:
+        """Runs the host planner into `plan` (pinned int32, at least cap words); returns the words
+        written.  The kv lengths order the tiles longest first and allow parts per tile; when
+        the workspace cannot hold the parts' partials, whole tiles (which need none) are planned."""
+        batch = h_qo.shape[0] - 1
         n_tiles, n_splits = ctypes.c_int32(), ctypes.c_int32()
         words, ws = ctypes.c_int64(), ctypes.c_int64()
-        # kv lengths order the tiles longest first
-        h_indptr = h_kv.to(torch.int64)
-        h_last = h_last32.to(torch.int64)
-        n_pages = h_indptr[1:] - h_indptr[:-1]
-        kv_len = torch.where(n_pages > 0, (n_pages - 1) * page_size + h_last, n_pages).to(torch.int32)
         for target in (target_workgroups, -1):
-            rc = L.dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, num_qo_heads, num_kv_heads,
-                                     head_dim, target, tiles.data_ptr(), cap, ctypes.byref(n_tiles),
-                                     ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
+            rc = _lib.lib().dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, self._hq, self._hkv,
+                                              self._d, target, plan.data_ptr(), cap, ctypes.byref(n_tiles),
+                                              ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
             _lib.check(rc, "prefill begin_forward")
-            # a workspace too small for the parts' partials: whole tiles need none
             if ws.value <= self._workspace.numel() * self._workspace.element_size():
                 break
-        self._batch, self._nnz, self._n_tiles, self._n_splits = batch, nnz, n_tiles.value, n_splits.value
-        self._tiles = staging.to_device(block, max(int(words.value), 4), paged_kv_indices.device)
+        self._batch, self._nnz = batch, (int(h_qo[-1]) if batch > 0 else 0)
+        self._n_tiles, self._n_splits = n_tiles.value, n_splits.value
+        return int(words.value)
+
+    def begin_forward_with_metadata(self, meta_words: int, fill_metadata, starts: dict,
+                                    qo_indptr_host: torch.Tensor, paged_kv_indptr_host: torch.Tensor,
+                                    paged_kv_last_page_len_host: torch.Tensor,
+                                    paged_kv_indices_host: torch.Tensor, num_qo_heads: int,
+                                    num_kv_heads: int, head_dim: int, page_size: int, device: torch.device,
+                                    target_workgroups: int = 0) -> torch.Tensor:
+        """begin_forward for callers that also have the step's other index arrays to upload
+        (the forward context): metadata and plan travel in ONE pinned block and ONE upload
+        kernel.  fill_metadata(view) writes the caller's meta_words int32 words (a multiple of
+        4) into the front of the block; starts maps "indptr", "kv_page_indptr",
+        "kv_page_indices" and "kv_last_page_lens" to their word offsets in it.  Returns the
+        device tensor that holds the metadata words (the caller slices its views)."""
+        if meta_words % 4:
+            raise ValueError("meta_words must be a multiple of 4 (16-byte alignment of the plan)")
+        self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
+        h_qo = qo_indptr_host.to(torch.int32).contiguous()
+        h_kv = paged_kv_indptr_host.to(torch.int32).contiguous()
+        h_last = paged_kv_last_page_len_host.to(torch.int32).contiguous()
+        cap, kv_len = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices_host, paged_kv_indices_host)
+        block = staging.take(meta_words + max(cap, 4))
+        fill_metadata(block.tensor[:meta_words])
+        words = self._plan_into(block.tensor[meta_words:], cap, h_qo, kv_len, target_workgroups)
+        dev = staging.to_device(block, meta_words + max(words, 4), device)
+        batch = h_qo.shape[0] - 1
+        used = int(h_kv[-1]) if batch > 0 else 0
+        self._tiles = dev[meta_words:]
+        self._qo_indptr = dev[starts["indptr"]: starts["indptr"] + batch + 1]
+        self._indptr = dev[starts["kv_page_indptr"]: starts["kv_page_indptr"] + batch + 1]
+        self._indices = dev[starts["kv_page_indices"]: starts["kv_page_indices"] + used]
+        self._last = dev[starts["kv_last_page_lens"]: starts["kv_last_page_lens"] + batch]
         self._planned = True
+        return dev[:meta_words]
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor, causal: bool = True,
                 sm_scale: Optional[float] = None, **_ignored) -> torch.Tensor:

@@ -342,6 +342,58 @@ def test_joined_prepare_equals_context_then_begin_forward():
     assert torch.equal(wl_a.pool.pages.view(torch.int16), wl_b.pool.pages.view(torch.int16))
 
 
+def test_joined_prefill_prepare_equals_context_then_begin_forward():
+    """FlashPrefillCtx.init_and_plan (metadata and plan in one pinned block, one upload kernel)
+    against init_paged_prefill_ctx + begin_forward: the same six arrays on the device, the same
+    plan (in parts per tile here: two chunks are few tiles), the same output bits."""
+    from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.model.context.flash import FlashPrefillCtx
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+    from deserve_amd.synthetic import fill_normal
+    from deserve_amd.task import SamplingParams, TaskData
+
+    print("[case] joined prefill prepare", flush=True)
+    prior, chunk = [1500, 37], [130, 64]
+    shape = dict(num_qo_heads=HQ, num_kv_heads=HKV, head_dim=D, page_size=P)
+    outs, ctxs, wrappers = [], [], []
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    q = torch.randn((sum(chunk), HQ, D), device=DEV, generator=gen).to(torch.bfloat16)
+    for joined in (False, True):
+        pool = GpuPagePool(1, 200, P, DEV, torch.bfloat16)
+        fill_normal(pool.pages, 77)
+        rows = PageTableAllocator(2, 4096, P, DEV)
+        tasks = [TaskData(f"j{b}", prior[b], 1, chunk[b], prior[b] + chunk[b], SamplingParams()) for b in range(2)]
+        caches = [PagedKVCache.empty(rows, pool) for _ in range(2)]
+        w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(32 << 20, dtype=torch.uint8, device=DEV))
+        if joined:
+            c = FlashPrefillCtx.init_and_plan(tasks, caches, w, **shape)
+        else:
+            c = FlashPrefillCtx.init_paged_prefill_ctx(tasks, caches, w)
+            w.begin_forward(qo_indptr=c.indptr, paged_kv_indptr=c.kv_page_indptr, paged_kv_indices=c.kv_page_indices,
+                            paged_kv_last_page_len=c.kv_last_page_lens, qo_indptr_host=c.host["indptr"],
+                            paged_kv_indptr_host=c.host["kv_page_indptr"],
+                            paged_kv_last_page_len_host=c.host["kv_last_page_lens"],
+                            paged_kv_indices_host=c.host["kv_page_indices"], **shape)
+        outs.append(w.forward(q, pool.pages[0], causal=True))
+        ctxs.append(c)
+        wrappers.append(w)
+    a, b = ctxs
+    for f in ("indptr", "kv_page_indices", "kv_page_indptr", "kv_last_page_lens", "offsets", "seqlens"):
+        assert torch.equal(getattr(a, f), getattr(b, f)), f
+        assert torch.equal(getattr(b, f).cpu(), b.host[f]), f
+    wa, wb = wrappers
+    assert (wa._n_tiles, wa._n_splits, wa._batch, wa._nnz) == (wb._n_tiles, wb._n_splits, wb._batch, wb._nnz)
+    assert wa._n_splits > 1
+    n = min(wa._tiles.numel(), wb._tiles.numel())
+    assert torch.equal(wa._tiles[:n], wb._tiles[:n])
+    for x, y in ((wb._qo_indptr, b.indptr), (wb._indptr, b.kv_page_indptr), (wb._indices, b.kv_page_indices),
+                 (wb._last, b.kv_last_page_lens)):
+        assert torch.equal(x, y)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
 def test_graphed_decode_step_on_the_generic_kernel_follows_the_item_count():
     """head_dim 64 takes the generic attention kernel, which is launched with one workgroup
     per work item: a captured launch is only valid for its item count.  Contexts grow by a
