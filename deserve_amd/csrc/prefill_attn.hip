@@ -788,15 +788,18 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
     }
     int32_t *p = plan_host;
     for (const Tile &t : tiles) {
-        // parts of equal length, in units of four 32-token blocks (the kernel's loop is
-        // unrolled by four); a part that starts past the tile's last block is empty
+        // Parts of equal length, in units of four 32-token blocks (the kernel's loop is
+        // unrolled by four), measured on the keys the tile sees under the causal mask; the
+        // last part is open-ended.  The parts are disjoint and cover all blocks, so they are
+        // also right without the mask (the last part then holds the rest of the request); a
+        // part that starts past what the tile sees is empty.
         const int64_t blocks = (t.keys + kBlock - 1) / kBlock;
         const int64_t chunk = ((blocks + splits - 1) / splits + 3) / 4 * 4;
         for (int s = 0; s < splits; s++) {
             *p++ = t.b;
             *p++ = t.row;
-            *p++ = splits > 1 ? (int32_t)std::min<int64_t>(s * chunk, (blocks + 3) / 4 * 4) : 0;
-            *p++ = splits > 1 && s + 1 < splits ? (int32_t)((s + 1) * chunk) : kWholeRange;
+            *p++ = (int32_t)(s * chunk);
+            *p++ = s + 1 < splits ? (int32_t)((s + 1) * chunk) : kWholeRange;
             *p++ = s;
         }
     }

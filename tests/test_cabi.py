@@ -234,7 +234,7 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
         blocks = -(-(4096 + row + 64) // 32)              # keys the tile's last row sees, in blocks
         begin, end = mine[:, 2].tolist(), mine[:, 3].tolist()
         assert begin[0] == 0 and all(x % 4 == 0 for x in begin) and end[-1] == 0x7fffffff
-        assert end[:-1] == begin[1:] and begin[-1] < blocks
+        assert end[:-1] == begin[1:] and begin[-1] < blocks and begin == sorted(set(begin))
     # the longest tile first
     assert t[0, 1] == 448
     # short keys limit the parts: a part holds at least 512 tokens
@@ -247,9 +247,14 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     assert _prefill_plan(lib, qo, kv_len, 32, 8, target=-1)[2] == 1
     big = np.array([0, 2048], np.int32)
     assert _prefill_plan(lib, big, np.array([4096], np.int32), 32, 8, target=256)[2] == 1
-    # a part past a tile's last block is empty: begin is clamped to the tile's blocks (rounded up to four)
+    # the parts of a tile are disjoint and cover every block, also past what the tile sees under
+    # the causal mask (a launch without the mask reads the rest of the request in the last part)
     qo2 = np.array([0, 64, 128], np.int32)
     rc, t, splits, parts, ws = _prefill_plan(lib, qo2, np.array([4096, 100], np.int32), 32, 8, target=256)
     assert splits == 8
     short = t[t[:, 0] == 1]
-    assert short[:, 2].tolist() == [0] + [4] * 7
+    assert short[:, 2].tolist() == [4 * i for i in range(8)]
+    assert short[:, 3].tolist() == [4 * i for i in range(1, 8)] + [0x7fffffff]
+    no_keys = _prefill_plan(lib, qo2, np.array([4096, 0], np.int32), 32, 8, target=256)[1]
+    none = no_keys[no_keys[:, 0] == 1]
+    assert none[:, 2].tolist() == [0] * 8 and none[:, 3].tolist() == [0] * 7 + [0x7fffffff]

@@ -298,7 +298,7 @@ def test_prefill_attention_random_shapes():
 
     rng = np.random.default_rng(77)
     w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device="cuda"))
-    done = 0
+    done, parts_seen = 0, set()
     while done < 40:
         P = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
         Hkv = int(rng.choice([1, 2, 4, 8]))
@@ -310,11 +310,14 @@ def test_prefill_attention_random_shapes():
         kv = [int(n + rng.integers(0, 300)) if rng.random() < 0.85 else int(rng.integers(0, n + 1)) for n in qo]
         if sum(qo) == 0:
             continue
+        if done % 5 == 4:          # every fifth case: long keys, so that the plan cuts the tiles into parts
+            kv[0] += int(rng.integers(1000, 3000))
         causal = bool(rng.integers(0, 2))
         _announce("prefill random", P, Hq, Hkv, dtype, kv, qo, causal)
         sc = make_scenario(2000 + done, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
         w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                         _dev_i32(sc.kv_last_page_lens), Hq, Hkv, 128, P)
+        parts_seen.add(w._n_splits)
         out = w.forward(to_torch(sc.q, dtype), to_torch(sc.pages, dtype), causal=causal)
         w.end_forward()
         torch.cuda.synchronize()
@@ -324,6 +327,7 @@ def test_prefill_attention_random_shapes():
         assert np.isfinite(got).all()
         assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (P, Hq, Hkv, dtype, kv, qo, causal)
         done += 1
+    assert 1 in parts_seen and max(parts_seen) >= 2, parts_seen
 
 
 def test_decode_attention_random_shapes():
