@@ -211,7 +211,8 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     for (long &pg : cur.page) pg = 0;
     auto fetch_page = [&]() {
         kv.page_ids = cur.page_ids;
-        if (kPageCoversTile) cur.page[0] = cur.page_ids[page_slot_of(kv, cur.t, cur.t_end)];
+        // an exhausted stream (t_end == 0) reads no block table: its descriptors are empty anyway
+        if (kPageCoversTile) cur.page[0] = cur.t_end > 0 ? cur.page_ids[page_slot_of(kv, cur.t, cur.t_end)] : 0;
         if (kPagesPerTile > 1) {
             // an exhausted stream (t_end == 0) keeps loading from page 0, which every pool has
 #pragma unroll

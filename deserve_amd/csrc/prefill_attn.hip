@@ -828,8 +828,9 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     using namespace dskv;
     DSKV_REQUIRE(batch >= 0 && nnz >= 0 && n_tiles >= 0, "prefill_attn: negative sizes");
     if (batch == 0 || nnz == 0) return 0;
-    DSKV_REQUIRE(out && q && qo_indptr && pages_layer && kv_page_indices && kv_page_indptr &&
-                     kv_last_page_len, "prefill_attn: null pointer argument");
+    // kv_page_indices may be null when no request has a page (it is only read for requests that do)
+    DSKV_REQUIRE(out && q && qo_indptr && pages_layer && kv_page_indptr && kv_last_page_len,
+                 "prefill_attn: null pointer argument");
     DSKV_REQUIRE(dtype == DSKV_F32 || dtype == DSKV_F16 || dtype == DSKV_BF16,
                  "prefill_attn: unknown dtype %d", dtype);
     DSKV_REQUIRE(n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0,

@@ -251,6 +251,7 @@ PREFILL_CASES = [
     ("long_tile", [900], [300], 16, 32, 8, 128, "bf16"),
     ("no_kv", [0, 40], [2, 8], 16, 32, 8, 128, "bf16"),
     ("more_queries_than_kv", [5, 33, 64], [9, 40, 64], 16, 32, 8, 128, "bf16"),
+    ("no_pages_at_all", [0, 0], [3, 70], 16, 32, 8, 128, "bf16"),      # an empty block table: rows of zeros
     # few tiles over long keys: planned in 4 and 8 parts per tile, most parts of the short requests empty
     ("split_parts", [5000, 1100, 40], [200, 130, 40], 16, 32, 8, 128, "bf16"),
     ("split_parts_f16_page8_group8", [3000, 2049], [65, 1], 8, 64, 8, 128, "f16"),
