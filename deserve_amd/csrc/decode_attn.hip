@@ -134,7 +134,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     // to its page yet.  The wave that will read it - kv head `kvh` of the item that ends
     // the request - writes its 256 bytes of K and of V first and waits until the cache
     // has them; nobody else reads that row in this launch.
-    if (k_new) {
+    auto append_new_rows = [&]() {
         for (int idx = item_begin; idx < item_end; idx++) {
             const Item it = load_item(idx);
             if (!it.tail) continue;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
                     *reinterpret_cast<const u32x4 *>(v_new + src + (lane - 16) * 8);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+    };
 
     // Q rows of one item as the B operand of the score MFMAs (zero beyond the group), and,
     // with a rope table, the cosines and sines of the lane's 16 dim pairs at the request's
@@ -254,9 +254,19 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     QRaw qnext;
     load_q(item_begin, qnext);
     settle();
+    // The new rows are written while the first tiles are already on their way (the chain item
+    // -> page id -> store -> acknowledgement then runs beside the first K/V loads instead of
+    // in front of them) - unless one of those tiles holds a new row: the first kStages tiles
+    // all belong to the workgroup's first item (items are padded to whole rounds of the
+    // ring), so that is the case only if that item ends its request within them.
+    const Item first_item = load_item(item_begin);
+    const bool rows_first =
+        k_new && first_item.tail && first_item.tok_end - 1 < first_item.tok_begin + kStages * kTile;
+    if (rows_first) append_new_rows();
     TileRegs ring[kStages];
 #pragma unroll
     for (int s = 0; s < kStages; s++) load_next(ring[s]);
+    if (k_new && !rows_first) append_new_rows();
 
     // ---- compute side
     for (int idx = item_begin; idx < item_end; idx++) {
