@@ -62,6 +62,12 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--section", choices=["swap", "fragmented", "prefill"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
+    ap.add_argument("--page-size", type=int, default=16,
+                    help="tokens per page of the benched pool (BASELINE's configurations use 16; the "
+                         "reference deploys with 8, worker_api.py:170)")
+    ap.add_argument("--prefill-one-chunk-only", action="store_true",
+                    help="with --section prefill: only the 512-token chunk over 4096 prior tokens "
+                         "(12 launches with parts, 12 with whole tiles), for profiler runs")
     ap.add_argument("--prefill-config4-only", action="store_true",
                     help="with --section prefill: only configuration 4's launches on its own data "
                          "(20 appends, 20 attention launches), for profiler runs whose per-kernel "
@@ -325,7 +331,7 @@ def swap_section(seed: int):
             "streams_run_beside_compute": independent}
 
 
-def prefill_section(seed: int, extras: bool = True):
+def prefill_section(seed: int, extras: bool = True, config4: bool = True):
     """Baseline configuration 4 (Llama-3-8B stage): 16 sequences each append a 512-token chunk
     at a start offset U[0,15] inside a partially filled page and attend over a prior context
     U[0,8192].  Timed per layer on the launch stream: the chunk append and the paged prefill
@@ -343,6 +349,50 @@ def prefill_section(seed: int, extras: bool = True):
 
     dev = torch.device("cuda")
     L, P, Hq, Hkv, D, B, n = 4, 16, 32, 8, 128, 16, 512
+
+    def one_chunk_measure(gen):
+        # One 512-token chunk over 4096 prior tokens: the step budget of the reference's scheduler
+        # (engine/pipeline/scheduler.py:74,85).  8 query tiles x 8 kv heads are 64 workgroups, so
+        # the plan cuts every tile's K/V range into parts (merged by a second pass); timed with
+        # that plan and with whole tiles.
+        one_prior = 4096
+        one_pool = GpuPagePool(2, (one_prior + n) // P + 8, P, dev, torch.bfloat16)
+        fill_normal(one_pool.pages, seed + 44)
+        one_rows = PageTableAllocator(1, one_prior + 1024, P, dev)
+        one_task = [TaskData("p_one", one_prior, 1, n, one_prior + n, SamplingParams())]
+        one_cache = [PagedKVCache.empty(one_rows, one_pool)]
+        one_w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
+        one_c = FlashPrefillCtx.init_paged_prefill_ctx(one_task, one_cache, one_w)
+        one_q = torch.randn((2, n, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
+        one_chunk = {}
+        for label, target in (("parts", 0), ("whole_tiles", -1)):
+            one_w.begin_forward(qo_indptr=one_c.indptr, paged_kv_indptr=one_c.kv_page_indptr,
+                                paged_kv_indices=one_c.kv_page_indices,
+                                paged_kv_last_page_len=one_c.kv_last_page_lens, num_qo_heads=Hq,
+                                num_kv_heads=Hkv, head_dim=D, page_size=P, qo_indptr_host=one_c.host["indptr"],
+                                paged_kv_indptr_host=one_c.host["kv_page_indptr"],
+                                paged_kv_last_page_len_host=one_c.host["kv_last_page_lens"],
+                                paged_kv_indices_host=one_c.host["kv_page_indices"], target_workgroups=target)
+            evs = []
+            for rep in range(12):
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                one_w.forward(one_q[rep % 2], one_pool.pages[rep % 2], causal=True)
+                e.record()
+                evs.append((s, e))
+            torch.cuda.synchronize()
+            ts = sorted(s.elapsed_time(e) for s, e in evs[2:])
+            one_chunk[label] = {"parts_per_tile": one_w._n_splits, "workgroups": one_w._n_tiles * Hkv,
+                                "us_per_layer": round(ts[len(ts) // 2] * 1e3, 1)}
+            one_w.end_forward()
+        one_flops = 4 * Hq * D * (n * one_prior + n * (n + 1) // 2)
+        for v in one_chunk.values():
+            v["TFLOPs"] = round(one_flops / v["us_per_layer"] / 1e6, 1)
+        return one_chunk
+
+    if not config4:
+        return {"one_512_token_chunk_over_4096":
+                one_chunk_measure(torch.Generator(device="cuda").manual_seed(seed + 43))}
     rng = np.random.default_rng(seed + 40)
     prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
     pool = GpuPagePool(L, int((-(-(prior + n) // P)).sum()) + 8, P, dev, torch.bfloat16)
@@ -404,43 +454,7 @@ def prefill_section(seed: int, extras: bool = True):
     pool.pages.zero_()
     attn_zero_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
     w.end_forward()
-    # One 512-token chunk over 4096 prior tokens: the step budget of the reference's scheduler
-    # (engine/pipeline/scheduler.py:74,85).  8 query tiles x 8 kv heads are 64 workgroups, so
-    # the plan cuts every tile's K/V range into parts (merged by a second pass); timed with
-    # that plan and with whole tiles.
-    one_prior = 4096
-    one_pool = GpuPagePool(2, (one_prior + n) // P + 8, P, dev, torch.bfloat16)
-    fill_normal(one_pool.pages, seed + 44)
-    one_rows = PageTableAllocator(1, one_prior + 1024, P, dev)
-    one_task = [TaskData("p_one", one_prior, 1, n, one_prior + n, SamplingParams())]
-    one_cache = [PagedKVCache.empty(one_rows, one_pool)]
-    one_w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(64 << 20, dtype=torch.uint8, device=dev))
-    one_c = FlashPrefillCtx.init_paged_prefill_ctx(one_task, one_cache, one_w)
-    one_q = torch.randn((2, n, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
-    one_chunk = {}
-    for label, target in (("parts", 0), ("whole_tiles", -1)):
-        one_w.begin_forward(qo_indptr=one_c.indptr, paged_kv_indptr=one_c.kv_page_indptr,
-                            paged_kv_indices=one_c.kv_page_indices,
-                            paged_kv_last_page_len=one_c.kv_last_page_lens, num_qo_heads=Hq,
-                            num_kv_heads=Hkv, head_dim=D, page_size=P, qo_indptr_host=one_c.host["indptr"],
-                            paged_kv_indptr_host=one_c.host["kv_page_indptr"],
-                            paged_kv_last_page_len_host=one_c.host["kv_last_page_lens"],
-                            paged_kv_indices_host=one_c.host["kv_page_indices"], target_workgroups=target)
-        evs = []
-        for rep in range(12):
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            one_w.forward(one_q[rep % 2], one_pool.pages[rep % 2], causal=True)
-            e.record()
-            evs.append((s, e))
-        torch.cuda.synchronize()
-        ts = sorted(s.elapsed_time(e) for s, e in evs[2:])
-        one_chunk[label] = {"parts_per_tile": one_w._n_splits, "workgroups": one_w._n_tiles * Hkv,
-                            "us_per_layer": round(ts[len(ts) // 2] * 1e3, 1)}
-        one_w.end_forward()
-    one_flops = 4 * Hq * D * (n * one_prior + n * (n + 1) // 2)
-    for v in one_chunk.values():
-        v["TFLOPs"] = round(one_flops / v["us_per_layer"] / 1e6, 1)
+    one_chunk = one_chunk_measure(gen)
     result.update({"attention_us_per_layer_zero_data": round(attn_zero_us, 1),
                    "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
                    "one_512_token_chunk_over_4096": one_chunk})
@@ -579,7 +593,8 @@ def main() -> int:
         import torch
         torch.cuda.set_device(0)
         if a.section == "prefill":
-            print(json.dumps(prefill_section(a.seed, extras=not a.prefill_config4_only)))
+            print(json.dumps(prefill_section(a.seed, extras=not a.prefill_config4_only,
+                                             config4=not a.prefill_one_chunk_only)))
         else:
             print(json.dumps({"swap": swap_section, "fragmented": fragmented_section}[a.section](a.seed)))
         return 0
@@ -600,7 +615,7 @@ def main() -> int:
     if not os.path.exists(_lib.LIB_PATH):
         _lib.build()
     torch.cuda.set_device(0)
-    L, Hq, Hkv, D, P = 16, 32, 8, 128, 16
+    L, Hq, Hkv, D, P = 16, 32, 8, 128, a.page_size
     graph_steps = 0 if a.no_graph else 24
     rope_steps = 0 if (a.rope or a.no_rope_step) else 24          # the step once more with rotation, as a model runs it
     total_steps = a.steps + a.warmup + graph_steps + rope_steps
@@ -723,8 +738,9 @@ def main() -> int:
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE.json configs[1]: Llama-3-8B stage, 16 layers, bf16, GQA 32q/8kv, "
-                               "head_dim 128, page 16, decode batch 64, ctx U[256,4096], scattered pages; "
+        "config": {"workload": ("BASELINE.json configs[1]" if P == 16 else "BASELINE.json configs[1] with another page size")
+                               + ": Llama-3-8B stage, 16 layers, bf16, GQA 32q/8kv, "
+                               f"head_dim 128, page {P}, decode batch 64, ctx U[256,4096], scattered pages; "
                                "step = host plan + 16 x (append 1 token + paged decode attention)"
                                + (" + RoPE" if a.rope else ""),
                    "batch": wl.batch, "layers": L, "kv_tokens": int(sum(t.start_pos for t in wl.tasks)),
@@ -745,7 +761,7 @@ def main() -> int:
         achieved = (sum(attn_bytes_layer) / len(attn_bytes_layer)) / (avg_ms * 1e-3) / 1e9
         traffic = traffic_workload = traffic_alg = None
         tfile = os.path.join(ROOT, "profiles", "decode_attn_cfg2_traffic.json")
-        if os.path.exists(tfile):
+        if os.path.exists(tfile) and P == 16:                # measured on the 16-token pages of configuration 2
             tj = json.load(open(tfile))
             traffic = tj.get("hbm_bytes_per_launch")
             traffic_workload, traffic_alg = tj.get("workload"), tj.get("algorithmic_bytes_per_launch")

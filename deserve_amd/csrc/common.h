@@ -50,8 +50,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // (max, sum): row r of `out` (rows x n_qo_heads x head_dim, of `dtype`) is merged from the
 // row_parts[2r + 1] parts that start at slot row_parts[2r]; rows with no parts are left
 // alone.  `wide`: eight waves per (row, head), for rows cut into dozens of parts.  Defined
-// beside the decode attention kernels, which write such partials; the prefill attention
-// kernel writes them too when its plan splits tiles.
+// beside the decode attention kernels, which write such partials.
 int launch_partials_merge(void *out, const float *part_o, const float *part_ml,
                           const int32_t *row_parts, int max_slots, int rows, int n_qo_heads,
                           int head_dim, int dtype, bool wide, hipStream_t stream);

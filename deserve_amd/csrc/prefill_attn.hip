@@ -27,7 +27,7 @@
 // A batch of few tiles (one 512-token chunk: 8 tiles x 8 kv heads) would leave most
 // of the chip idle.  The plan then cuts every tile's K/V range into parts; a part is
 // a workgroup of its own that leaves (maximum, sum, unnormalised O) of its rows in a
-// workspace, and the merge pass of the decode path turns the parts into the output.
+// workspace, and a merge pass (one workgroup per query row) turns the parts into the output.
 #include "kv_tile.h"
 
 #include <vector>
@@ -185,8 +185,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const u32x4 ones = {one2, one2, one2, one2};
 
     // A plan that splits tiles: every part leaves (max, sum, unnormalised O) of its rows in
-    // slot row * n_splits + split of the workspace, laid out as the merge pass of the decode
-    // path reads it; a part that sees nothing leaves zeros and a maximum below any real one.
+    // slot row * n_splits + split of the workspace (O blocks of all slots, then their (max,
+    // sum) pairs); a part that sees nothing leaves zeros and a maximum below any real one.
     auto store_partial = [&](int ct, float m, float l) {
         const long slot = (long)(q_begin + qrow[ct]) * n_splits + split;
         if (slot >= max_slots) return;   // a slot beyond the workspace is never written
@@ -684,6 +684,58 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
     }
 }
 
+// Merge pass of a plan in parts: output row r, head qh = sum_i w_i O_i / sum_i w_i l_i over
+// the n_splits partials of the row (slots r * n_splits + i), w_i = exp2(m_i - max_j m_j).
+// One workgroup per query row; a thread owns 16 consecutive dims of one head and requests
+// all of its parts' values at once (no block table, no lookup: the slots follow from the
+// row).  The decode path's merge kernel, launched with one wave per (row, head) and a table
+// of parts per row, took 11.5 us for the 512 rows of a chunk; this one takes about half.
+template <int DT, int kParts>
+__global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
+    uint16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
+    int n_qo_heads)
+{
+    typedef Elt<DT> E;
+    const long row = blockIdx.x;
+    for (int idx = threadIdx.x; idx < n_qo_heads * (kHeadDim / 16); idx += blockDim.x) {
+        const int qh = idx / (kHeadDim / 16), d0 = (idx % (kHeadDim / 16)) * 16;
+        f32x4 o[kParts][4];
+        float m[kParts], l[kParts];
+#pragma unroll
+        for (int i = 0; i < kParts; i++) {
+            const long slot = row * kParts + i;
+            const float *src = part_o + (slot * n_qo_heads + qh) * kHeadDim + d0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[i][j] = *reinterpret_cast<const f32x4 *>(src + 4 * j);
+            const float *ml = part_ml + (slot * n_qo_heads + qh) * 2;
+            m[i] = ml[0];
+            l[i] = ml[1];
+        }
+        float m_all = m[0];
+#pragma unroll
+        for (int i = 1; i < kParts; i++) m_all = fmaxf(m_all, m[i]);
+        f32x4 acc[4] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f},
+                        f32x4{0.f, 0.f, 0.f, 0.f}};
+        float l_all = 0.f;
+#pragma unroll
+        for (int i = 0; i < kParts; i++) {
+            const float w = __builtin_amdgcn_exp2f(m[i] - m_all);
+            l_all += w * l[i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] += w * o[i][j];
+        }
+        const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+        uint16_t *dst = out + (row * n_qo_heads + qh) * kHeadDim + d0;
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+            const u32x4 w4 = {E::pack2(acc[j][0] * inv, acc[j][1] * inv), E::pack2(acc[j][2] * inv, acc[j][3] * inv),
+                              E::pack2(acc[j + 1][0] * inv, acc[j + 1][1] * inv),
+                              E::pack2(acc[j + 1][2] * inv, acc[j + 1][3] * inv)};
+            *reinterpret_cast<u32x4 *>(dst + 4 * j) = w4;
+        }
+    }
+}
+
 static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads)
 {
     const int group = n_qo_heads / n_kv_heads;
@@ -719,8 +771,8 @@ extern "C" int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz)
     using namespace dskv;
     if (batch < 0 || nnz < 0) return 0;
     // entries: one per tile, or per part of a tile when the plan splits (then there are few
-    // tiles: at most 2 * kMaxSplitTarget parts); then two words per query row
-    return kTileWords * ((int64_t)batch + nnz + 2 * kMaxSplitTarget) + 2 * nnz;
+    // tiles: at most 2 * kMaxSplitTarget parts)
+    return kTileWords * ((int64_t)batch + nnz + 2 * kMaxSplitTarget);
 }
 
 extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
@@ -780,7 +832,7 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
         }
     }
     const int64_t n_entries = (int64_t)tiles.size() * splits;
-    const int64_t words = n_entries * kTileWords + (splits > 1 ? 2 * nnz : 0);
+    const int64_t words = n_entries * kTileWords;
     if (words > capacity_words) {
         set_error("prefill_plan: plan needs %lld words, buffer has %lld", (long long)words,
                   (long long)capacity_words);
@@ -803,11 +855,6 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
             *p++ = s;
         }
     }
-    if (splits > 1)
-        for (int64_t r = 0; r < nnz; r++) {
-            *p++ = (int32_t)(r * splits);
-            *p++ = splits;
-        }
     *n_tiles_out = (int32_t)n_entries;
     *n_splits_out = splits;
     *plan_words_out = words;
@@ -884,9 +931,26 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
         }
 #undef DSKV_LAUNCH_PREFILL
         DSKV_LAUNCH_CHECK("prefill_attn_mfma_kernel");
-        if (n_splits > 1)   // the parts' partials become the output rows
-            return launch_partials_merge(out, part_o, part_ml, plan_dev + (int64_t)n_tiles * kTileWords,
-                                         (int)max_slots, nnz, n_qo_heads, head_dim, dtype, false, s);
+        if (n_splits > 1) {   // the parts' partials become the output rows
+#define DSKV_LAUNCH_PARTS(DT, N)                                                                 \
+    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>), dim3((unsigned)nnz), dim3(256), 0, s, \
+                       (uint16_t *)out, part_o, part_ml, n_qo_heads)
+#define DSKV_LAUNCH_PARTS_N(DT)                                                  \
+    switch (n_splits) {                                                          \
+    case 2: DSKV_LAUNCH_PARTS(DT, 2); break;                                     \
+    case 3: DSKV_LAUNCH_PARTS(DT, 3); break;                                     \
+    case 4: DSKV_LAUNCH_PARTS(DT, 4); break;                                     \
+    case 5: DSKV_LAUNCH_PARTS(DT, 5); break;                                     \
+    case 6: DSKV_LAUNCH_PARTS(DT, 6); break;                                     \
+    case 7: DSKV_LAUNCH_PARTS(DT, 7); break;                                     \
+    default: DSKV_LAUNCH_PARTS(DT, 8); break;                                    \
+    }
+            if (dtype == DSKV_BF16) DSKV_LAUNCH_PARTS_N(DSKV_BF16)
+            else DSKV_LAUNCH_PARTS_N(DSKV_F16)
+#undef DSKV_LAUNCH_PARTS_N
+#undef DSKV_LAUNCH_PARTS
+            DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
+        }
     } else {
         dim3 grid((unsigned)nnz, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_GEN(DT)                                                                      \

@@ -160,7 +160,7 @@ def test_decode_plan_rejects_bad_metadata_and_small_buffers():
 
 
 def _prefill_plan(lib, qo, kv_len, hq, hkv, target=0, head_dim=128, cap=None):
-    """Runs dskv_prefill_plan; returns (rc, entries (n, 5), n_splits, row parts or None, workspace bytes)."""
+    """Runs dskv_prefill_plan; returns (rc, entries (n, 5), n_splits, None, workspace bytes)."""
     batch, nnz = len(qo) - 1, int(qo[-1])
     cap = lib.dskv_prefill_plan_bound(batch, nnz) if cap is None else cap
     plan = np.zeros(max(cap, 8), np.int32)
@@ -172,9 +172,8 @@ def _prefill_plan(lib, qo, kv_len, hq, hkv, target=0, head_dim=128, cap=None):
     if rc:
         return rc, None, None, None, None
     entries = plan[: 5 * n.value].reshape(-1, 5)
-    parts = plan[5 * n.value: words.value].reshape(-1, 2) if splits.value > 1 else None
-    assert words.value == 5 * n.value + (0 if parts is None else 2 * nnz)
-    return rc, entries, splits.value, parts, ws.value
+    assert words.value == 5 * n.value
+    return rc, entries, splits.value, None, ws.value
 
 
 def test_prefill_plan_tiles_cover_all_query_rows():
@@ -218,8 +217,7 @@ def test_prefill_plan_with_kv_lengths_orders_tiles_longest_first():
 def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     """One 512-token chunk over 4096 prior tokens is 8 tiles x 8 kv heads = 64 workgroups: for
     256 it is planned in 4 parts per tile.  The parts of a tile are consecutive block ranges
-    that start at multiples of four blocks and cover [0, blocks of the tile); every query row
-    gets its run of slots; a full batch, a plan without lengths or with another head dim,
+    that start at multiples of four blocks and cover [0, blocks of the tile); a full batch, a plan without lengths or with another head dim,
     and target < 0 are not split."""
     lib = _lib.lib()
     qo = np.array([0, 512], np.int32)
@@ -227,7 +225,6 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     rc, t, splits, parts, ws = _prefill_plan(lib, qo, kv_len, 32, 8, target=256)
     assert rc == 0 and splits == 4 and len(t) == 8 * 4
     assert ws == 512 * 4 * 32 * (128 + 2) * 4
-    assert parts.tolist() == [[r * 4, 4] for r in range(512)]
     for row in range(0, 512, 64):
         mine = t[t[:, 1] == row]
         assert mine[:, 0].tolist() == [0] * 4 and mine[:, 4].tolist() == [0, 1, 2, 3]
