@@ -76,6 +76,7 @@ __device__ __forceinline__ int padded_end(const Item &it)
 
 // Position of the load side in this workgroup's tile stream (wave-uniform).
 struct LoadCursor {
+    Item ahead;                // item next_item, requested when the item before it was entered
     int next_item, item_end;   // next item to enter, one past the workgroup's last
     int t, t_end, t_pad_end;   // next tile, valid end and padded end of the current item
     const_i32_ptr page_ids;    // current item's block table
@@ -206,6 +207,7 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     LoadCursor cur;
     cur.next_item = item_begin;
     cur.item_end = item_end;
+    cur.ahead = load_item(item_begin);
     cur.t = cur.t_end = cur.t_pad_end = 0;
     cur.page_ids = indices_c;
     for (long &pg : cur.page) pg = 0;
@@ -224,7 +226,11 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     };
     auto settle = [&]() {   // step into following items until a tile is available (or none is left)
         while (cur.t >= cur.t_pad_end && cur.next_item < cur.item_end) {
-            const Item it = load_item(cur.next_item++);
+            // the item's words were requested an item ago: entering it costs no round trip in
+            // front of the page id; the request for the one after it goes out now
+            const Item it = cur.ahead;
+            cur.next_item++;
+            cur.ahead = load_item(min(cur.next_item, cur.item_end - 1));
             cur.t = it.tok_begin;
             cur.t_end = it.tok_end;
             cur.t_pad_end = padded_end(it);
@@ -269,8 +275,10 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     if (k_new && !rows_first) append_new_rows();
 
     // ---- compute side
+    Item item_ahead = load_item(item_begin);
     for (int idx = item_begin; idx < item_end; idx++) {
-        const Item item = load_item(idx);
+        const Item item = item_ahead;
+        item_ahead = load_item(min(idx + 1, item_end - 1));   // for the next turn, like its q rows
         const int t_end = item.tok_end;
         // Q of the following item: issued now, so that it is older than every
         // tile load still in flight when it is needed (no drain at the switch)
