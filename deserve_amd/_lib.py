@@ -16,6 +16,17 @@ LIB_PATH = os.path.join(_HERE, "libdskv.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 F32, F16, BF16 = 0, 1, 2
+ABI_VERSION = 3          # DSKV_ABI_VERSION of the include/dskv.h these signatures were written against
+
+
+class MixedPlanInfo(ctypes.Structure):
+    """dskv_mixed_plan_t of include/dskv.h."""
+    _fields_ = [("n_tiles", c_int32), ("n_splits", c_int32), ("n_tile_rows", c_int32),
+                ("n_decode_rows", c_int32), ("n_decode_items", c_int32), ("n_decode_workgroups", c_int32),
+                ("plan_words", c_int64), ("decode_plan_at", c_int64), ("row_map_at", c_int64),
+                ("tile_rows_at", c_int64), ("tile_workspace_bytes", c_int64),
+                ("decode_workspace_bytes", c_int64)]
+
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -63,6 +74,13 @@ _SIGNATURES = {
                                     c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_int64, c_int32,
                                     c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
                                     c_int32, c_void_p]),
+    "dskv_mixed_plan_bound": (c_int64, [c_int32, c_int64, c_int64]),
+    "dskv_mixed_plan": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
+                                  c_int32, c_int32, c_int32, c_void_p, c_int64, POINTER(MixedPlanInfo)]),
+    "dskv_mixed_attn": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, POINTER(MixedPlanInfo), c_void_p, c_int64,
+                                  c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float,
+                                  c_int32, c_int32, c_void_p]),
     "dskv_apply_rope": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_int32, c_int32, c_int32, c_int32, c_int32, c_float, c_int32,
                                   c_void_p]),
@@ -111,6 +129,9 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
+        if handle.dskv_version() != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} has ABI version {handle.dskv_version()}, this binding was written "
+                               f"against {ABI_VERSION}: rebuild the library (its argument lists differ)")
         _lib = handle
     return _lib
 

@@ -51,9 +51,33 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // row_parts[2r + 1] parts that start at slot row_parts[2r]; rows with no parts are left
 // alone.  `wide`: eight waves per (row, head), for rows cut into dozens of parts.  Defined
 // beside the decode attention kernels, which write such partials.
+// row_map (may be null): request r's output row is row_map[r] instead of r.
 int launch_partials_merge(void *out, const float *part_o, const float *part_ml,
-                          const int32_t *row_parts, int max_slots, int rows, int n_qo_heads,
-                          int head_dim, int dtype, bool wide, hipStream_t stream);
+                          const int32_t *row_parts, const int32_t *row_map, int max_slots, int rows,
+                          int n_qo_heads, int head_dim, int dtype, bool wide, hipStream_t stream);
+
+// The split-KV decode path for requests that are rows of a ragged batch (the one-row
+// requests of a prefill batch): request i has `len` kv tokens, its block table starts at
+// entry `page_begin` of the table array, and its query and output are row `row` of q and out.
+// plan_decode_rows is dskv_decode_plan over such a list (same plan layout, the items name the
+// rows); decode_rows_attn is dskv_decode_attn over that plan, with row_map[i] = reqs[i].row on
+// the device for the merge pass.  decode_mfma_shape: whether the 16-bit decode kernel takes
+// the shape (the routing is only worth it then).
+struct DecodeRow {
+    int64_t len;
+    int32_t page_begin, row;
+};
+int plan_decode_rows(const DecodeRow *reqs, int32_t batch, int32_t n_qo_heads, int32_t head_dim,
+                     int32_t target_workgroups, int32_t *plan_host, int64_t plan_capacity_words,
+                     int32_t *n_items_out, int32_t *n_workgroups_out, int64_t *plan_words_out,
+                     int64_t *workspace_bytes_out);
+int decode_rows_attn(void *out, const void *q, const void *pages_layer,
+                     const int32_t *kv_page_indices, const int32_t *plan_dev, int32_t n_items,
+                     int32_t n_workgroups, void *workspace, int64_t workspace_bytes, int32_t n_rows,
+                     const int32_t *row_map, int32_t n_qo_heads, int32_t n_kv_heads,
+                     int32_t head_dim, int32_t page_size, float sm_scale, int32_t dtype,
+                     hipStream_t stream);
+bool decode_mfma_shape(int head_dim, int n_qo_heads, int n_kv_heads, int page_size);
 
 static inline bool is_pow2(int64_t x) { return x > 0 && (x & (x - 1)) == 0; }
 static inline int ilog2(int64_t x) {

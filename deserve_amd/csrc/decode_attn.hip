@@ -61,7 +61,8 @@ constexpr int kMinTilesPerWorkgroup = DSKV_DECODE_MIN_TILES;
 // Work item written by the planner.  slot < 0: the item covers its whole request
 // and writes the final output row; otherwise it writes partial slot `slot`.
 struct Item {
-    int32_t b, tok_begin, tok_end, slot;
+    int32_t b;            // row of q and of the output (the request's index in a decode batch)
+    int32_t tok_begin, tok_end, slot;
     int32_t page_begin;   // kv_page_indptr[b]: start of the request's block table
     int32_t tail;         // 1: tok_end is the request's length (the item holds its newest token)
     int32_t reserved[2];
@@ -263,11 +264,19 @@ __global__ __launch_bounds__(64 * kMaxWaves, DSKV_DECODE_MIN_WAVES) void decode_
     // The new rows are written while the first tiles are already on their way (the chain item
     // -> page id -> store -> acknowledgement then runs beside the first K/V loads instead of
     // in front of them) - unless one of those tiles holds a new row: the first kStages tiles
-    // all belong to the workgroup's first item (items are padded to whole rounds of the
-    // ring), so that is the case only if that item ends its request within them.
-    const Item first_item = load_item(item_begin);
-    const bool rows_first =
-        k_new && first_item.tail && first_item.tok_end - 1 < first_item.tok_begin + kStages * kTile;
+    // all belong to the workgroup's first item with tiles (items are padded to whole rounds of
+    // the ring), so that is the case only if that item ends its request within them.
+    // A request without tokens is an item without tiles (it only writes a zero row): the load
+    // side steps over it, so "first" means the first item that has tiles.
+    bool rows_first = false;
+    if (k_new) {
+        for (int idx = item_begin; idx < item_end; idx++) {
+            const Item it = load_item(idx);
+            if (it.tok_end <= it.tok_begin) continue;
+            rows_first = it.tail && it.tok_end - 1 < it.tok_begin + kStages * kTile;
+            break;
+        }
+    }
     if (rows_first) append_new_rows();
     TileRegs ring[kStages];
 #pragma unroll
@@ -486,7 +495,8 @@ __global__ __launch_bounds__(64) void decode_attn_generic_kernel(
 template <int DT, int kWaves>
 __global__ __launch_bounds__(64 * kWaves) void decode_merge_kernel(
     void *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
-    const int32_t *__restrict__ req_parts, int max_slots, int n_qo_heads, int head_dim)
+    const int32_t *__restrict__ req_parts, const int32_t *__restrict__ row_map, int max_slots,
+    int n_qo_heads, int head_dim)
 {
     typedef LoadElt<DT> L;
     constexpr int kBatch = 8;   // O rows in flight per round
@@ -497,6 +507,9 @@ __global__ __launch_bounds__(64 * kWaves) void decode_merge_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int first = req_parts[2 * b], n = req_parts[2 * b + 1];
     if (n <= 0) return;   // written directly by the attention kernel
+    // the output row of request b: b itself in a decode batch, an entry of the row map when
+    // the requests are the one-row members of a ragged batch
+    const long out_row = row_map ? row_map[b] : b;
     if (first < 0 || first + n > max_slots) return;
     const float *ml_base = part_ml + ((long)first * n_qo_heads + qh) * 2;
     const float *o_base = part_o + ((long)first * n_qo_heads + qh) * head_dim;
@@ -568,8 +581,14 @@ __global__ __launch_bounds__(64 * kWaves) void decode_merge_kernel(
 #pragma unroll
     for (int k = 0; k < 4; k++) {
         const int d = lane + 64 * k;
-        if (d < head_dim) L::put(out, ((long)b * n_qo_heads + qh) * head_dim + d, acc[k] * inv);
+        if (d < head_dim) L::put(out, (out_row * n_qo_heads + qh) * head_dim + d, acc[k] * inv);
     }
+}
+
+bool decode_mfma_shape(int head_dim, int n_qo_heads, int n_kv_heads, int page_size)
+{
+    return head_dim == kHeadDim && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0 &&
+           n_qo_heads / n_kv_heads <= 16 && is_pow2(page_size);
 }
 
 static bool mfma_path(int dtype, int head_dim, int n_qo_heads, int n_kv_heads)
@@ -608,41 +627,20 @@ extern "C" int64_t dskv_decode_plan_bound(int32_t batch, int64_t total_tokens)
     return kPlanHeaderWords + max_items * kItemWords + (kMaxWorkgroups + 1) + (int64_t)batch * 2;
 }
 
-extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
-                                const int32_t *kv_last_page_len_host, int32_t batch,
-                                int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
-                                int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
-                                int64_t plan_capacity_words, int32_t *n_items_out,
-                                int32_t *n_workgroups_out, int64_t *plan_words_out,
-                                int64_t *workspace_bytes_out)
-{
-    using namespace dskv;
-    DSKV_REQUIRE(batch >= 0, "decode_plan: negative batch");
-    DSKV_REQUIRE(n_items_out && n_workgroups_out && plan_words_out && workspace_bytes_out,
-                 "decode_plan: null output pointer");
-    DSKV_REQUIRE(page_size > 0 && n_qo_heads > 0 && n_kv_heads > 0 && head_dim > 0 &&
-                     n_qo_heads % n_kv_heads == 0,
-                 "decode_plan: bad shape (page %d, heads %d/%d, dim %d)", page_size, n_qo_heads,
-                 n_kv_heads, head_dim);
-    *n_items_out = 0;
-    *n_workgroups_out = 0;
-    *plan_words_out = 0;
-    *workspace_bytes_out = 0;
-    if (batch == 0) return 0;
-    DSKV_REQUIRE(kv_page_indptr_host && kv_last_page_len_host && plan_host,
-                 "decode_plan: null pointer argument");
+namespace dskv {
 
-    std::vector<int64_t> len(batch), tiles(batch);
+// The planner proper.  reqs[i]: tokens, start of the block table and q / output row of
+// request i (row i itself for a decode batch).
+int plan_decode_rows(const DecodeRow *reqs, int32_t batch, int32_t n_qo_heads, int32_t head_dim,
+                     int32_t target_workgroups, int32_t *plan_host, int64_t plan_capacity_words,
+                     int32_t *n_items_out, int32_t *n_workgroups_out, int64_t *plan_words_out,
+                     int64_t *workspace_bytes_out)
+{
+    std::vector<int64_t> tiles(batch);
     int64_t total_tiles = 0;
     for (int b = 0; b < batch; b++) {
-        const int64_t np = (int64_t)kv_page_indptr_host[b + 1] - kv_page_indptr_host[b];
-        DSKV_REQUIRE(np >= 0, "decode_plan: kv_page_indptr not monotone at %d", b);
-        const int32_t last = kv_last_page_len_host[b];
-        DSKV_REQUIRE(np == 0 || (last >= 1 && last <= page_size),
-                     "decode_plan: kv_last_page_len[%d] = %d outside [1, %d]", b, last, page_size);
-        len[b] = np > 0 ? (np - 1) * page_size + last : 0;
-        DSKV_REQUIRE(len[b] < (int64_t(1) << 30), "decode_plan: request %d too long", b);
-        tiles[b] = (len[b] + kTile - 1) / kTile;
+        DSKV_REQUIRE(reqs[b].len >= 0 && reqs[b].len < (int64_t(1) << 30), "decode_plan: request %d too long", b);
+        tiles[b] = (reqs[b].len + kTile - 1) / kTile;
         total_tiles += tiles[b];
     }
     // Workgroup count: one per CU unless told otherwise, fewer when there is so
@@ -660,8 +658,9 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
     int64_t w = 0, g0 = 0;                        // current workgroup, global tile index
     auto share_end = [&](int64_t wg) { return (wg + 1) * total_tiles / wgs; };
     for (int b = 0; b < batch; b++) {
+        const int64_t len = reqs[b].len;
         if (tiles[b] == 0) {
-            items.push_back(Item{b, 0, 0, -1, kv_page_indptr_host[b], 0, {0, 0}});
+            items.push_back(Item{reqs[b].row, 0, 0, -1, reqs[b].page_begin, 0, {0, 0}});
             continue;
         }
         const size_t first_item = items.size();
@@ -673,9 +672,9 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
             }
             const int64_t room = (w + 1 < wgs) ? share_end(w) - g0 : tiles[b] - done;
             const int64_t take = std::min(room, tiles[b] - done);
-            items.push_back(Item{b, (int32_t)(done * kTile),
-                                 (int32_t)std::min<int64_t>((done + take) * kTile, len[b]), -1,
-                                 kv_page_indptr_host[b], done + take == tiles[b], {0, 0}});
+            items.push_back(Item{reqs[b].row, (int32_t)(done * kTile),
+                                 (int32_t)std::min<int64_t>((done + take) * kTile, len), -1,
+                                 reqs[b].page_begin, done + take == tiles[b], {0, 0}});
             done += take;
             g0 += take;
         }
@@ -715,6 +714,45 @@ extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
     return 0;
 }
 
+}  // namespace dskv
+
+extern "C" int dskv_decode_plan(const int32_t *kv_page_indptr_host,
+                                const int32_t *kv_last_page_len_host, int32_t batch,
+                                int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
+                                int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
+                                int64_t plan_capacity_words, int32_t *n_items_out,
+                                int32_t *n_workgroups_out, int64_t *plan_words_out,
+                                int64_t *workspace_bytes_out)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(batch >= 0, "decode_plan: negative batch");
+    DSKV_REQUIRE(n_items_out && n_workgroups_out && plan_words_out && workspace_bytes_out,
+                 "decode_plan: null output pointer");
+    DSKV_REQUIRE(page_size > 0 && n_qo_heads > 0 && n_kv_heads > 0 && head_dim > 0 &&
+                     n_qo_heads % n_kv_heads == 0,
+                 "decode_plan: bad shape (page %d, heads %d/%d, dim %d)", page_size, n_qo_heads,
+                 n_kv_heads, head_dim);
+    *n_items_out = 0;
+    *n_workgroups_out = 0;
+    *plan_words_out = 0;
+    *workspace_bytes_out = 0;
+    if (batch == 0) return 0;
+    DSKV_REQUIRE(kv_page_indptr_host && kv_last_page_len_host && plan_host,
+                 "decode_plan: null pointer argument");
+    std::vector<DecodeRow> reqs(batch);
+    for (int b = 0; b < batch; b++) {
+        const int64_t np = (int64_t)kv_page_indptr_host[b + 1] - kv_page_indptr_host[b];
+        DSKV_REQUIRE(np >= 0, "decode_plan: kv_page_indptr not monotone at %d", b);
+        const int32_t last = kv_last_page_len_host[b];
+        DSKV_REQUIRE(np == 0 || (last >= 1 && last <= page_size),
+                     "decode_plan: kv_last_page_len[%d] = %d outside [1, %d]", b, last, page_size);
+        reqs[b] = DecodeRow{np > 0 ? (np - 1) * page_size + last : 0, kv_page_indptr_host[b], b};
+    }
+    return plan_decode_rows(reqs.data(), batch, n_qo_heads, head_dim, target_workgroups, plan_host,
+                            plan_capacity_words, n_items_out, n_workgroups_out, plan_words_out,
+                            workspace_bytes_out);
+}
+
 namespace dskv {
 
 // k_new / v_new non-null: the fused form, which also writes the step's token of every
@@ -725,7 +763,8 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
                             int64_t workspace_bytes, int32_t batch, int32_t n_qo_heads,
                             int32_t n_kv_heads, int32_t head_dim, int32_t page_size,
                             float sm_scale, int32_t dtype, int32_t phases, void *stream,
-                            const void *k_new, const void *v_new, const float *rope_table)
+                            const void *k_new, const void *v_new, const float *rope_table,
+                            const int32_t *row_map = nullptr)
 {
     DSKV_REQUIRE(phases >= 1 && phases <= 3, "decode_attn: phases must be 1, 2 or 3");
     DSKV_REQUIRE(batch >= 0 && n_items >= 0 && n_workgroups >= 0,
@@ -814,25 +853,37 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
         // One wave needs a round trip per 8 parts, eight waves a barrier and a second pass
         // through LDS: they break even at about 32 parts.
         const bool wide = (int64_t)n_items > 32 * (int64_t)batch;
-        return launch_partials_merge(out, part_o, part_ml, req_parts, (int)max_slots, batch, n_qo_heads,
-                                     head_dim, dtype, wide, s);
+        return launch_partials_merge(out, part_o, part_ml, req_parts, row_map, (int)max_slots, batch,
+                                     n_qo_heads, head_dim, dtype, wide, s);
     }
     return 0;
 }
 
+int decode_rows_attn(void *out, const void *q, const void *pages_layer,
+                     const int32_t *kv_page_indices, const int32_t *plan_dev, int32_t n_items,
+                     int32_t n_workgroups, void *workspace, int64_t workspace_bytes, int32_t n_rows,
+                     const int32_t *row_map, int32_t n_qo_heads, int32_t n_kv_heads,
+                     int32_t head_dim, int32_t page_size, float sm_scale, int32_t dtype,
+                     hipStream_t stream)
+{
+    return decode_attn_impl(out, q, pages_layer, kv_page_indices, plan_dev, n_items, n_workgroups,
+                            workspace, workspace_bytes, n_rows, n_qo_heads, n_kv_heads, head_dim,
+                            page_size, sm_scale, dtype, 3, stream, nullptr, nullptr, nullptr, row_map);
+}
+
 int launch_partials_merge(void *out, const float *part_o, const float *part_ml,
-                          const int32_t *row_parts, int max_slots, int rows, int n_qo_heads,
-                          int head_dim, int dtype, bool wide, hipStream_t s)
+                          const int32_t *row_parts, const int32_t *row_map, int max_slots, int rows,
+                          int n_qo_heads, int head_dim, int dtype, bool wide, hipStream_t s)
 {
     dim3 grid((unsigned)rows, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_MERGE(DT)                                                                     \
     do {                                                                                          \
         if (wide)                                                                                 \
             hipLaunchKernelGGL((decode_merge_kernel<DT, 8>), grid, dim3(512), 0, s, out, part_o,  \
-                               part_ml, row_parts, max_slots, n_qo_heads, head_dim);              \
+                               part_ml, row_parts, row_map, max_slots, n_qo_heads, head_dim);     \
         else                                                                                      \
             hipLaunchKernelGGL((decode_merge_kernel<DT, 1>), grid, dim3(64), 0, s, out, part_o,   \
-                               part_ml, row_parts, max_slots, n_qo_heads, head_dim);              \
+                               part_ml, row_parts, row_map, max_slots, n_qo_heads, head_dim);     \
     } while (0)
     if (dtype == DSKV_F32) DSKV_LAUNCH_MERGE(DSKV_F32);
     else if (dtype == DSKV_F16) DSKV_LAUNCH_MERGE(DSKV_F16);

@@ -20,4 +20,7 @@ void set_error(const char *fmt, ...)
 }  // namespace dskv
 
 extern "C" const char *dskv_last_error(void) { return dskv::g_error; }
-extern "C" int dskv_version(void) { return 1; }
+// Bumped whenever an exported signature changes (2: num_pages argument of the append entry
+// points, kv lengths / parts in the prefill plan; 3: plans that route one-row requests of a
+// prefill batch to the decode kernel).
+extern "C" int dskv_version(void) { return DSKV_ABI_VERSION; }

@@ -444,8 +444,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
             // is the whole point of requesting them early.  Nothing else needs the fences here:
             // the loop of this path writes LDS through these loads only, and the LDS reads of
             // the previous iteration have been consumed.
+            // (the empty statements pin the compiler's order of ordinary LDS accesses around the
+            // barrier, which the builtin by itself does not: the previous iteration's operand
+            // reads stay above it, this iteration's below)
             DSKV_WAIT_VMEM(3 * kRowGroups);
+            asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
         } else {
             __syncthreads();
         }
@@ -693,10 +698,12 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
 template <int DT, int kParts>
 __global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
     uint16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
-    int n_qo_heads)
+    const int32_t *__restrict__ rows, int n_qo_heads)
 {
     typedef Elt<DT> E;
-    const long row = blockIdx.x;
+    // rows (may be null): the query rows that were computed in parts, when they are not all
+    // rows of the batch (the others were left to the decode kernel)
+    const long row = rows ? rows[blockIdx.x] : blockIdx.x;
     for (int idx = threadIdx.x; idx < n_qo_heads * (kHeadDim / 16); idx += blockDim.x) {
         const int qh = idx / (kHeadDim / 16), d0 = (idx % (kHeadDim / 16)) * 16;
         f32x4 o[kParts][4];
@@ -775,25 +782,16 @@ extern "C" int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz)
     return kTileWords * ((int64_t)batch + nnz + 2 * kMaxSplitTarget);
 }
 
-extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
-                                 int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads,
-                                 int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
-                                 int64_t capacity_words, int32_t *n_tiles_out,
-                                 int32_t *n_splits_out, int64_t *plan_words_out,
-                                 int64_t *workspace_bytes_out)
+namespace dskv {
+
+// The tile planner.  skip (may be null): requests marked there get no tiles (their single
+// row is computed by the decode kernel).
+static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host, const char *skip,
+                      int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                      int32_t target_workgroups, int32_t *plan_host, int64_t capacity_words,
+                      int32_t *n_tiles_out, int32_t *n_splits_out, int64_t *plan_words_out,
+                      int64_t *workspace_bytes_out)
 {
-    using namespace dskv;
-    DSKV_REQUIRE(batch >= 0 && n_tiles_out && n_splits_out && plan_words_out && workspace_bytes_out,
-                 "prefill_plan: bad arguments");
-    DSKV_REQUIRE(n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0,
-                 "prefill_plan: n_qo_heads %d not a multiple of n_kv_heads %d", n_qo_heads,
-                 n_kv_heads);
-    *n_tiles_out = 0;
-    *n_splits_out = 1;
-    *plan_words_out = 0;
-    *workspace_bytes_out = 0;
-    if (batch == 0) return 0;
-    DSKV_REQUIRE(qo_indptr_host && plan_host, "prefill_plan: null pointer argument");
     const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads);
     // later query tiles of a request see more keys: they come first within a request
     struct Tile { int32_t b, row; int64_t keys; };
@@ -803,6 +801,7 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
         const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
         DSKV_REQUIRE(n_b >= 0, "prefill_plan: qo_indptr not monotone at %d", b);
         nnz += n_b;
+        if (skip && skip[b]) continue;
         for (int64_t i = (n_b + rows - 1) / rows - 1; i >= 0; i--) {
             const int64_t last_row = std::min<int64_t>(i * rows + rows, n_b) - 1;
             const int64_t keys = kv_len_host ? std::max<int64_t>((int64_t)kv_len_host[b] - n_b + last_row + 1, 0) : 0;
@@ -863,16 +862,141 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
     return 0;
 }
 
-extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr,
-                                 const void *pages_layer, const int32_t *kv_page_indices,
-                                 const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
-                                 const int32_t *plan_dev, int32_t n_tiles, int32_t n_splits,
-                                 void *workspace, int64_t workspace_bytes, int32_t batch,
-                                 int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
-                                 int32_t head_dim, int32_t page_size, float sm_scale,
-                                 int32_t causal, int32_t dtype, void *stream)
+}  // namespace dskv
+
+extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
+                                 int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads,
+                                 int32_t head_dim, int32_t target_workgroups, int32_t *plan_host,
+                                 int64_t capacity_words, int32_t *n_tiles_out,
+                                 int32_t *n_splits_out, int64_t *plan_words_out,
+                                 int64_t *workspace_bytes_out)
 {
     using namespace dskv;
+    DSKV_REQUIRE(batch >= 0 && n_tiles_out && n_splits_out && plan_words_out && workspace_bytes_out,
+                 "prefill_plan: bad arguments");
+    DSKV_REQUIRE(n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0,
+                 "prefill_plan: n_qo_heads %d not a multiple of n_kv_heads %d", n_qo_heads,
+                 n_kv_heads);
+    *n_tiles_out = 0;
+    *n_splits_out = 1;
+    *plan_words_out = 0;
+    *workspace_bytes_out = 0;
+    if (batch == 0) return 0;
+    DSKV_REQUIRE(qo_indptr_host && plan_host, "prefill_plan: null pointer argument");
+    return plan_tiles(qo_indptr_host, kv_len_host, nullptr, batch, n_qo_heads, n_kv_heads, head_dim,
+                      target_workgroups, plan_host, capacity_words, n_tiles_out, n_splits_out,
+                      plan_words_out, workspace_bytes_out);
+}
+
+// ---------------------------------------------------------------------------
+// Mixed batches: one-row requests to the decode kernel, the others to query tiles
+// ---------------------------------------------------------------------------
+extern "C" int64_t dskv_mixed_plan_bound(int32_t batch, int64_t nnz, int64_t total_kv_tokens)
+{
+    if (batch < 0 || nnz < 0 || total_kv_tokens < 0) return 0;
+    // tile entries, padding, the decode plan, the row map and the list of tiled rows
+    return dskv_prefill_plan_bound(batch, nnz) + 4 + dskv_decode_plan_bound(batch, total_kv_tokens) +
+           (int64_t)batch + nnz + 8;
+}
+
+extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_page_indptr_host,
+                               const int32_t *kv_last_page_len_host, int32_t batch,
+                               int32_t page_size, int32_t n_qo_heads, int32_t n_kv_heads,
+                               int32_t head_dim, int32_t target_workgroups,
+                               int32_t route_one_row_requests, int32_t *plan_host,
+                               int64_t capacity_words, dskv_mixed_plan_t *info)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(info, "mixed_plan: null info pointer");
+    *info = dskv_mixed_plan_t{};
+    info->n_splits = 1;
+    DSKV_REQUIRE(batch >= 0, "mixed_plan: negative batch");
+    DSKV_REQUIRE(page_size > 0 && n_qo_heads > 0 && n_kv_heads > 0 && head_dim > 0 &&
+                     n_qo_heads % n_kv_heads == 0,
+                 "mixed_plan: bad shape (page %d, heads %d/%d, dim %d)", page_size, n_qo_heads,
+                 n_kv_heads, head_dim);
+    if (batch == 0) return 0;
+    DSKV_REQUIRE(qo_indptr_host && kv_page_indptr_host && kv_last_page_len_host && plan_host,
+                 "mixed_plan: null pointer argument");
+    // One query row under the end-aligned mask sees every kv token of its request, with or
+    // without the mask: exactly a decode row.  Routed only where the 16-bit decode kernel
+    // takes the shape; a request without kv tokens stays with the tiles (a row of zeros).
+    const bool route = route_one_row_requests && decode_mfma_shape(head_dim, n_qo_heads, n_kv_heads, page_size);
+    std::vector<int32_t> kv_len(batch);
+    std::vector<char> routed(batch, 0);
+    std::vector<DecodeRow> rows;
+    std::vector<int32_t> tile_rows;
+    for (int b = 0; b < batch; b++) {
+        const int64_t np = (int64_t)kv_page_indptr_host[b + 1] - kv_page_indptr_host[b];
+        DSKV_REQUIRE(np >= 0, "mixed_plan: kv_page_indptr not monotone at %d", b);
+        const int32_t last = kv_last_page_len_host[b];
+        DSKV_REQUIRE(np == 0 || (last >= 1 && last <= page_size),
+                     "mixed_plan: kv_last_page_len[%d] = %d outside [1, %d]", b, last, page_size);
+        const int64_t len = np > 0 ? (np - 1) * page_size + last : 0;
+        DSKV_REQUIRE(len < (int64_t(1) << 30), "mixed_plan: request %d too long", b);
+        kv_len[b] = (int32_t)len;
+        const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
+        DSKV_REQUIRE(n_b >= 0, "mixed_plan: qo_indptr not monotone at %d", b);
+        if (route && n_b == 1 && len > 0) {
+            routed[b] = 1;
+            rows.push_back(DecodeRow{len, kv_page_indptr_host[b], qo_indptr_host[b]});
+        } else {
+            for (int64_t i = 0; i < n_b; i++) tile_rows.push_back((int32_t)(qo_indptr_host[b] + i));
+        }
+    }
+    int64_t tile_words = 0;
+    int rc = plan_tiles(qo_indptr_host, kv_len.data(), rows.empty() ? nullptr : routed.data(), batch,
+                        n_qo_heads, n_kv_heads, head_dim, target_workgroups, plan_host, capacity_words,
+                        &info->n_tiles, &info->n_splits, &tile_words, &info->tile_workspace_bytes);
+    if (rc) return rc;
+    info->tile_workspace_bytes = (info->tile_workspace_bytes + 255) / 256 * 256;
+    info->n_tile_rows = (int32_t)tile_rows.size();
+    int64_t at = (tile_words + 3) / 4 * 4;
+    info->plan_words = tile_words;
+    if (rows.empty()) return 0;
+    info->decode_plan_at = at;
+    int64_t decode_words = 0;
+    if (at > capacity_words) at = capacity_words;   // the decode planner then reports the shortage
+    rc = plan_decode_rows(rows.data(), (int32_t)rows.size(), n_qo_heads, head_dim, target_workgroups,
+                          plan_host + at, capacity_words - at, &info->n_decode_items,
+                          &info->n_decode_workgroups, &decode_words, &info->decode_workspace_bytes);
+    if (rc) return rc;
+    info->n_decode_rows = (int32_t)rows.size();
+    at += decode_words;
+    const int64_t total = at + (int64_t)rows.size() + (int64_t)tile_rows.size();
+    if (total > capacity_words) {
+        set_error("mixed_plan: plan needs %lld words, buffer has %lld", (long long)total,
+                  (long long)capacity_words);
+        return DSKV_E_NOMEM;
+    }
+    info->row_map_at = at;
+    for (const DecodeRow &r : rows) plan_host[at++] = r.row;
+    info->tile_rows_at = at;
+    std::copy(tile_rows.begin(), tile_rows.end(), plan_host + at);
+    info->plan_words = total;
+    return 0;
+}
+
+namespace dskv {
+
+static bool prefill_mfma_path(int dtype, int head_dim, int n_qo_heads, int n_kv_heads, float scale_log2)
+{
+    // the MFMA kernel takes maxima before scaling: it needs a positive, sane scale
+    return (dtype == DSKV_BF16 || dtype == DSKV_F16) && head_dim == kHeadDim && n_kv_heads > 0 &&
+           n_qo_heads / n_kv_heads <= kWaveCols && scale_log2 > 1e-6f && scale_log2 < 1e6f;
+}
+
+// merge_rows / n_merge_rows: the query rows the tiles cover when they are not all nnz rows of
+// the batch (null: all of them); an MFMA-path call with n_tiles == 0 then has nothing to do.
+static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
+                             const void *pages_layer, const int32_t *kv_page_indices,
+                             const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
+                             const int32_t *plan_dev, int32_t n_tiles, int32_t n_splits,
+                             void *workspace, int64_t workspace_bytes, int32_t batch, int32_t nnz,
+                             int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                             int32_t page_size, float sm_scale, int32_t causal, int32_t dtype,
+                             void *stream, const int32_t *merge_rows, int32_t n_merge_rows)
+{
     DSKV_REQUIRE(batch >= 0 && nnz >= 0 && n_tiles >= 0, "prefill_attn: negative sizes");
     if (batch == 0 || nnz == 0) return 0;
     // kv_page_indices may be null when no request has a page (it is only read for requests that do)
@@ -889,9 +1013,8 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     DSKV_REQUIRE(n_qo_heads <= 65535, "prefill_attn: too many heads");
     const float scale_log2 = sm_scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
-    // the MFMA kernel takes maxima before scaling: it needs a positive, sane scale
-    const bool mfma = (dtype == DSKV_BF16 || dtype == DSKV_F16) && head_dim == kHeadDim &&
-                      n_qo_heads / n_kv_heads <= kWaveCols && scale_log2 > 1e-6f && scale_log2 < 1e6f;
+    const bool mfma = prefill_mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads, scale_log2);
+    if (mfma && merge_rows && n_tiles == 0) return 0;   // every row went to the decode kernel
     if (mfma) {
         DSKV_REQUIRE(plan_dev && n_tiles > 0, "prefill_attn: missing plan");
         DSKV_REQUIRE(n_splits >= 1 && n_splits <= kMaxPrefillSplits && n_tiles % n_splits == 0,
@@ -933,8 +1056,9 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
         DSKV_LAUNCH_CHECK("prefill_attn_mfma_kernel");
         if (n_splits > 1) {   // the parts' partials become the output rows
 #define DSKV_LAUNCH_PARTS(DT, N)                                                                 \
-    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>), dim3((unsigned)nnz), dim3(256), 0, s, \
-                       (uint16_t *)out, part_o, part_ml, n_qo_heads)
+    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>),                                     \
+                       dim3((unsigned)(merge_rows ? n_merge_rows : nnz)), dim3(256), 0, s,      \
+                       (uint16_t *)out, part_o, part_ml, merge_rows, n_qo_heads)
 #define DSKV_LAUNCH_PARTS_N(DT)                                                  \
     switch (n_splits) {                                                          \
     case 2: DSKV_LAUNCH_PARTS(DT, 2); break;                                     \
@@ -949,7 +1073,7 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
             else DSKV_LAUNCH_PARTS_N(DSKV_F16)
 #undef DSKV_LAUNCH_PARTS_N
 #undef DSKV_LAUNCH_PARTS
-            DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
+            if (!merge_rows || n_merge_rows > 0) DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
         }
     } else {
         dim3 grid((unsigned)nnz, (unsigned)n_qo_heads);
@@ -964,4 +1088,72 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
         DSKV_LAUNCH_CHECK("prefill_attn_generic_kernel");
     }
     return 0;
+}
+
+}  // namespace dskv
+
+extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr,
+                                 const void *pages_layer, const int32_t *kv_page_indices,
+                                 const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
+                                 const int32_t *plan_dev, int32_t n_tiles, int32_t n_splits,
+                                 void *workspace, int64_t workspace_bytes, int32_t batch,
+                                 int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
+                                 int32_t head_dim, int32_t page_size, float sm_scale,
+                                 int32_t causal, int32_t dtype, void *stream)
+{
+    return dskv::prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
+                                   kv_last_page_len, plan_dev, n_tiles, n_splits, workspace,
+                                   workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
+                                   page_size, sm_scale, causal, dtype, stream, nullptr, 0);
+}
+
+extern "C" int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indptr,
+                               const void *pages_layer, const int32_t *kv_page_indices,
+                               const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
+                               const int32_t *plan_dev, const dskv_mixed_plan_t *info,
+                               void *workspace, int64_t workspace_bytes, int32_t batch, int32_t nnz,
+                               int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                               int32_t page_size, float sm_scale, int32_t causal, int32_t dtype,
+                               void *stream)
+{
+    using namespace dskv;
+    DSKV_REQUIRE(info, "mixed_attn: null plan info");
+    DSKV_REQUIRE(info->n_decode_rows >= 0 && info->n_tile_rows >= 0 && info->n_tiles >= 0 &&
+                     info->tile_workspace_bytes >= 0 && info->decode_workspace_bytes >= 0,
+                 "mixed_attn: negative sizes in the plan info");
+    const bool routed = info->n_decode_rows > 0;
+    const float scale_log2 = sm_scale * 1.4426950408889634f;
+    // Shapes and types outside the 16-bit kernels: the generic kernel computes every row
+    // of the batch by itself, routed or not.
+    const bool mfma = n_qo_heads > 0 && n_kv_heads > 0 && n_qo_heads % n_kv_heads == 0 &&
+                      prefill_mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads, scale_log2);
+    if (!routed || !mfma)
+        return prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
+                                 kv_last_page_len, plan_dev, info->n_tiles, info->n_splits, workspace,
+                                 workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
+                                 page_size, sm_scale, causal, dtype, stream, nullptr, 0);
+    DSKV_REQUIRE(plan_dev, "mixed_attn: missing plan");
+    DSKV_REQUIRE(info->n_decode_rows + info->n_tile_rows == nnz && info->n_decode_rows <= batch,
+                 "mixed_attn: the plan covers %d + %d rows, the batch has %d", info->n_decode_rows,
+                 info->n_tile_rows, nnz);
+    DSKV_REQUIRE(workspace_bytes >= info->tile_workspace_bytes + info->decode_workspace_bytes &&
+                     (workspace || info->tile_workspace_bytes + info->decode_workspace_bytes == 0),
+                 "mixed_attn: the plan needs a workspace of %lld bytes, got %lld",
+                 (long long)(info->tile_workspace_bytes + info->decode_workspace_bytes),
+                 (long long)workspace_bytes);
+    // The one-row requests: the split-KV decode pass (each K/V byte read once, at the speed
+    // of memory) and its merge; their partials lie behind those of the tile parts.
+    int rc = decode_rows_attn(out, q, pages_layer, kv_page_indices, plan_dev + info->decode_plan_at,
+                              info->n_decode_items, info->n_decode_workgroups,
+                              workspace ? (char *)workspace + info->tile_workspace_bytes : nullptr,
+                              workspace ? workspace_bytes - info->tile_workspace_bytes : 0,
+                              info->n_decode_rows, plan_dev + info->row_map_at, n_qo_heads, n_kv_heads,
+                              head_dim, page_size, sm_scale, dtype, (hipStream_t)stream);
+    if (rc) return rc;
+    // The others: query tiles (and the merge of their parts, over the tiled rows only).
+    return prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
+                             kv_last_page_len, plan_dev, info->n_tiles, info->n_splits, workspace,
+                             info->tile_workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
+                             page_size, sm_scale, causal, dtype, stream, plan_dev + info->tile_rows_at,
+                             info->n_tile_rows);
 }

@@ -44,11 +44,13 @@ struct dskv_swap {
     struct IdStretch {
         int64_t begin, end;
         hipEvent_t done[2];            // per direction stream that read it (null = unused)
+        bool sealed;                   // every reader's end has been recorded in `done`
     };
     std::deque<IdStretch> ids_pending; // oldest first
     std::vector<hipEvent_t> spare_events;
     bool probed = false;               // streams checked against the caller's compute stream
     bool independent = false;          // ... and found to run beside it
+    bool streams_exported = false;     // a caller holds the raw stream handles (dskv_swap_streams)
 };
 
 namespace dskv {
@@ -101,6 +103,9 @@ static void retire_ids(dskv_swap *h)
 {
     while (!h->ids_pending.empty()) {
         dskv_swap::IdStretch &st = h->ids_pending.front();
+        // a stretch whose call did not get as far as recording the end of its readers is
+        // only given up by wait_all, which drains both streams
+        if (!st.sealed) return;
         for (hipEvent_t e : st.done)
             if (e && hipEventQuery(e) != hipSuccess) {
                 (void)hipGetLastError();   // hipErrorNotReady is not a failure
@@ -149,7 +154,7 @@ static int stage_ids(dskv_swap *h, const int32_t *ids, int32_t n, hipStream_t s,
     std::copy(ids, ids + n, host);
     int rc = dskv_upload_words(dev, host, n, s);
     if (rc) return rc;
-    h->ids_pending.push_back(dskv_swap::IdStretch{begin, begin + len, {nullptr, nullptr}});
+    h->ids_pending.push_back(dskv_swap::IdStretch{begin, begin + len, {nullptr, nullptr}, false});
     h->ids_head = begin + len;
     *dev_out = dev;
     return 0;
@@ -167,6 +172,30 @@ static int release_ids_after(dskv_swap *h, int dir)
     DSKV_HIP(hipEventRecord(st.done[dir], h->stream[dir]));
     return 0;
 }
+
+// From stage_ids to the end of a call the newest stretch belongs to that call.  A call that
+// ends well seals it (the end of every reader is on record in `done`); one that fails on the
+// way has already enqueued the id upload and perhaps gather / scatter kernels that read the
+// stretch, so the guard records the end of whatever both streams hold now and seals it - or,
+// if even that fails, leaves it unsealed, which keeps the stretch (and the pinned mirror
+// behind it) out of circulation until dskv_swap_wait has drained the streams.
+struct IdsGuard {
+    dskv_swap *h;
+    bool armed;
+    void seal()
+    {
+        h->ids_pending.back().sealed = true;
+        armed = false;
+    }
+    ~IdsGuard()
+    {
+        if (!armed || h->ids_pending.empty()) return;
+        bool ok = true;
+        for (int dir = 0; dir < 2; dir++) ok = release_ids_after(h, dir) == 0 && ok;
+        (void)hipGetLastError();
+        h->ids_pending.back().sealed = ok;
+    }
+};
 
 // The gather and scatter kernels index the pool by page id: ids outside a layer are
 // refused here, on the host.
@@ -231,8 +260,10 @@ static int runs_beside(hipStream_t a, hipStream_t b, hipEvent_t ea, hipEvent_t e
     DSKV_HIP(hipStreamSynchronize(a));
     DSKV_HIP(hipStreamSynchronize(b));
     hipLaunchKernelGGL(idle_kernel, dim3(1), dim3(64), 0, a, ticks);
+    DSKV_LAUNCH_CHECK("idle_kernel");
     DSKV_HIP(hipEventRecord(ea, a));
     hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, b);
+    DSKV_LAUNCH_CHECK("empty_kernel");
     DSKV_HIP(hipEventRecord(eb, b));
     DSKV_HIP(hipEventSynchronize(eb));
     const hipError_t q = hipEventQuery(ea);       // still idling = b did not wait for a
@@ -353,6 +384,7 @@ extern "C" int dskv_swap_out_async(dskv_swap_t *h, void *host_dst, const void *p
     int32_t *ids_dev = nullptr;
     hipStream_t s = h->stream[0];
     if ((rc = stage_ids(h, page_ids_host, n_pages, s, &ids_dev))) return rc;
+    IdsGuard ids_guard{h, true};
     if ((rc = open_direction(h, 0, (hipStream_t)after_stream, s))) return rc;
     for (int64_t r0 = 0; r0 < rows; r0 += rows_per_chunk) {
         const int64_t r1 = std::min(rows, r0 + rows_per_chunk);
@@ -362,7 +394,9 @@ extern "C" int dskv_swap_out_async(dskv_swap_t *h, void *host_dst, const void *p
         DSKV_HIP(hipMemcpyAsync((char *)host_dst + r0 * page_bytes, h->staging[0],
                                 (size_t)((r1 - r0) * page_bytes), hipMemcpyDeviceToHost, s));
     }
-    return close_direction(h, 0);
+    if ((rc = close_direction(h, 0))) return rc;
+    ids_guard.seal();
+    return 0;
 }
 
 extern "C" int dskv_swap_in_async(dskv_swap_t *h, void *pool, const void *host_src,
@@ -384,6 +418,7 @@ extern "C" int dskv_swap_in_async(dskv_swap_t *h, void *pool, const void *host_s
     int32_t *ids_dev = nullptr;
     hipStream_t s = h->stream[1];
     if ((rc = stage_ids(h, page_ids_host, n_pages, s, &ids_dev))) return rc;
+    IdsGuard ids_guard{h, true};
     if ((rc = open_direction(h, 1, (hipStream_t)after_stream, s))) return rc;
     for (int64_t r0 = 0; r0 < rows; r0 += rows_per_chunk) {
         const int64_t r1 = std::min(rows, r0 + rows_per_chunk);
@@ -393,7 +428,9 @@ extern "C" int dskv_swap_in_async(dskv_swap_t *h, void *pool, const void *host_s
                                      layer_stride_bytes, page_bytes, r0, r1, s)))
             return rc;
     }
-    return close_direction(h, 1);
+    if ((rc = close_direction(h, 1))) return rc;
+    ids_guard.seal();
+    return 0;
 }
 
 extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const void *host_src,
@@ -418,6 +455,7 @@ extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const vo
     int32_t *ids_dev = nullptr;
     hipStream_t so = h->stream[0], si = h->stream[1];
     if ((rc = stage_ids(h, page_ids_host, n_pages, so, &ids_dev))) return rc;
+    IdsGuard ids_guard{h, true};
     if ((rc = open_direction(h, 0, (hipStream_t)after_stream, so))) return rc;
     if ((rc = open_direction(h, 1, (hipStream_t)after_stream, so))) return rc;
     // host_dst == host_src is a round trip through one buffer (two microbatch
@@ -443,7 +481,9 @@ extern "C" int dskv_swap_exchange_async(dskv_swap_t *h, void *host_dst, const vo
             return rc;
     }
     if ((rc = close_direction(h, 0))) return rc;
-    return close_direction(h, 1);
+    if ((rc = close_direction(h, 1))) return rc;
+    ids_guard.seal();
+    return 0;
 }
 
 extern "C" int dskv_swap_streams(dskv_swap_t *h, void **out_stream, void **in_stream)
@@ -451,6 +491,7 @@ extern "C" int dskv_swap_streams(dskv_swap_t *h, void **out_stream, void **in_st
     DSKV_REQUIRE(h && out_stream && in_stream, "swap_streams: null argument");
     *out_stream = h->stream[0];
     *in_stream = h->stream[1];
+    h->streams_exported = true;
     return 0;
 }
 
@@ -459,6 +500,13 @@ extern "C" int dskv_swap_bind_compute_stream(dskv_swap_t *h, void *compute_strea
 {
     using namespace dskv;
     DSKV_REQUIRE(h, "swap_bind_compute_stream: null handle");
+    if (h->streams_exported) {
+        // binding replaces streams that serialise with the compute stream, which would
+        // destroy handles a caller already holds
+        set_error("swap_bind_compute_stream: the engine's streams have been handed out "
+                  "(dskv_swap_streams); bind before asking for them");
+        return DSKV_E_STATE;
+    }
     int rc = wait_all(h);
     if (rc) return rc;
     hipStream_t compute = (hipStream_t)compute_stream;

@@ -96,6 +96,7 @@ class _PagedWrapper:
         self._planned = False
         self._rope_table, self._rope_key = None, None
         self._max_page_id = -1
+        self._empty_requests = []
 
     def _shape_args(self, num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int) -> None:
         self._hq, self._hkv, self._d, self._p = num_qo_heads, num_kv_heads, head_dim, page_size
@@ -210,6 +211,9 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
             raise RuntimeError(f"decode workspace too small: need {ws.value} bytes")
         self._batch, self._n_items, self._n_workgroups = batch, n_items.value, n_wgs.value
         self._rope_table, self._rope_key = None, None     # positions change with the step
+        # requests without a page: the fused append has no slot to write their token to
+        n_pages = h_indptr[1:] - h_indptr[:-1]
+        self._empty_requests = [int(b) for b in (n_pages <= 0).nonzero().flatten()[:4]] if batch > 0 else []
         return int(words.value)
 
     def begin_forward_with_metadata(self, meta_words: int, fill_metadata, indptr_at: int, indices_at: int,
@@ -276,6 +280,11 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
         if k_append is not None or v_append is not None:
             if k_append is None or v_append is None or phases not in (1, 3):
                 raise ValueError("the fused form takes both k_append and v_append, with the attention pass")
+            if self._empty_requests:
+                # the appended token is the request's last one (model/layer/attention.py:175-185):
+                # every request of the plan owns at least the page that holds it
+                raise ValueError(f"k_append / v_append: request(s) {self._empty_requests} have no page "
+                                 "(kv length 0 after the append); extend the caches before begin_forward")
             k_append, v_append = k_append.contiguous(), v_append.contiguous()
             want = (self._batch, self._hkv, self._d)
             if tuple(k_append.shape) != want or tuple(v_append.shape) != want or \
@@ -318,6 +327,12 @@ class BatchDecodeWithPagedKVCacheWrapper(_PagedWrapper):
 
 
 class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
+    """begin_forward plans on the host: requests with one query row (the decode rows of a
+    mixed step, which the reference sends through this wrapper together with the chunk:
+    engine/microbatch/processor.py:116-145) become split-KV decode work, the others query
+    tiles; forward (once per layer) launches the decode pass for the former and the tile
+    pass for the latter, both writing their rows of the same ragged output."""
+
     def begin_forward(self, qo_indptr: torch.Tensor, paged_kv_indptr: torch.Tensor,
                       paged_kv_indices: torch.Tensor, paged_kv_last_page_len: torch.Tensor,
                       num_qo_heads: int, num_kv_heads: int, head_dim: int, page_size: int, *,
@@ -325,29 +340,32 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
                       paged_kv_indptr_host: Optional[torch.Tensor] = None,
                       paged_kv_last_page_len_host: Optional[torch.Tensor] = None,
                       paged_kv_indices_host: Optional[torch.Tensor] = None,
-                      target_workgroups: int = 0, **_ignored) -> None:
+                      target_workgroups: int = 0, route_one_row_requests: bool = True,
+                      **_ignored) -> None:
         """The *_host arguments are host copies of the index tensors (the planner and the
         checks of the block tables run on the host; without them the device tensors are read
         back, which synchronises).
         target_workgroups: a batch of few query tiles (a chunk of a few hundred tokens) is
         planned in several parts per tile, merged by a second pass, so that the launch has
         about this many workgroups (0: one per compute unit; negative: never split); the parts'
-        partials go to the workspace buffer."""
+        partials go to the workspace buffer.
+        route_one_row_requests: False keeps one-row requests on the tile path (one live row
+        of a 64-row tile each), as for a plan of dskv_prefill_plan."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
         h_qo = self._host(qo_indptr, qo_indptr_host)
         h_kv = self._host(paged_kv_indptr, paged_kv_indptr_host)
         h_last = self._host(paged_kv_last_page_len, paged_kv_last_page_len_host)
-        cap, kv_len = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices, paged_kv_indices_host)
+        cap = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices, paged_kv_indices_host)
         block = staging.take(max(cap, 4))
-        words = self._plan_into(block.tensor, cap, h_qo, kv_len, target_workgroups)
+        words = self._plan_into(block.tensor, cap, h_qo, h_kv, h_last, target_workgroups, route_one_row_requests)
         self._tiles = staging.to_device(block, max(words, 4), paged_kv_indices.device)
         self._planned = True
 
     def _check_and_bound(self, h_qo: torch.Tensor, h_kv: torch.Tensor, h_last: torch.Tensor,
                          indices: torch.Tensor, indices_host: Optional[torch.Tensor]):
-        """Host-side checks of the index arrays; returns (words the plan may need, kv lengths)."""
+        """Host-side checks of the index arrays; returns the words the plan may need."""
         batch = h_qo.shape[0] - 1
         if batch > 0 and (int(h_qo[0]) != 0 or bool((h_qo[1:] < h_qo[:-1]).any())):
             raise ValueError("qo_indptr must start at 0 and not decrease")
@@ -355,37 +373,37 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
             raise ValueError("qo_indptr and paged_kv_indptr disagree about the batch")
         self._check_block_tables(h_kv, indices, indices_host, h_last)
         nnz = int(h_qo[-1]) if batch > 0 else 0
-        h_indptr = h_kv.to(torch.int64)
-        n_pages = h_indptr[1:] - h_indptr[:-1]
-        kv_len = torch.where(n_pages > 0, (n_pages - 1) * self._p + h_last[:max(batch, 0)].to(torch.int64),
-                             n_pages).to(torch.int32)
-        return int(_lib.lib().dskv_prefill_plan_bound(batch, nnz)), kv_len
+        total_tokens = int(h_kv[-1]) * self._p if batch > 0 else 0
+        return int(_lib.lib().dskv_mixed_plan_bound(batch, nnz, total_tokens))
 
-    def _plan_into(self, plan: torch.Tensor, cap: int, h_qo: torch.Tensor, kv_len: torch.Tensor,
-                   target_workgroups: int) -> int:
+    def _plan_into(self, plan: torch.Tensor, cap: int, h_qo: torch.Tensor, h_kv: torch.Tensor,
+                   h_last: torch.Tensor, target_workgroups: int, route: bool = True) -> int:
         """Runs the host planner into `plan` (pinned int32, at least cap words); returns the words
         written.  The kv lengths order the tiles longest first and allow parts per tile; when
-        the workspace cannot hold the parts' partials, whole tiles (which need none) are planned."""
+        the workspace cannot hold the parts' partials, whole tiles (which need none) are planned,
+        and if it cannot even hold the partials of cut decode rows, nothing is routed."""
         batch = h_qo.shape[0] - 1
-        n_tiles, n_splits = ctypes.c_int32(), ctypes.c_int32()
-        words, ws = ctypes.c_int64(), ctypes.c_int64()
-        for target in (target_workgroups, -1):
-            rc = _lib.lib().dskv_prefill_plan(h_qo.data_ptr(), kv_len.data_ptr(), batch, self._hq, self._hkv,
-                                              self._d, target, plan.data_ptr(), cap, ctypes.byref(n_tiles),
-                                              ctypes.byref(n_splits), ctypes.byref(words), ctypes.byref(ws))
+        info = _lib.MixedPlanInfo()
+        ws_bytes = self._workspace.numel() * self._workspace.element_size()
+        for target, routed in ((target_workgroups, route), (-1, route), (-1, False)):
+            rc = _lib.lib().dskv_mixed_plan(h_qo.data_ptr(), h_kv.data_ptr(), h_last.data_ptr(), batch,
+                                            self._p, self._hq, self._hkv, self._d, target, int(routed),
+                                            plan.data_ptr(), cap, ctypes.byref(info))
             _lib.check(rc, "prefill begin_forward")
-            if ws.value <= self._workspace.numel() * self._workspace.element_size():
+            if info.tile_workspace_bytes + info.decode_workspace_bytes <= ws_bytes:
                 break
         self._batch, self._nnz = batch, (int(h_qo[-1]) if batch > 0 else 0)
-        self._n_tiles, self._n_splits = n_tiles.value, n_splits.value
-        return int(words.value)
+        self._info = info
+        self._n_tiles, self._n_splits = info.n_tiles, info.n_splits
+        self._n_decode_rows = info.n_decode_rows
+        return int(info.plan_words)
 
     def begin_forward_with_metadata(self, meta_words: int, fill_metadata, starts: dict,
                                     qo_indptr_host: torch.Tensor, paged_kv_indptr_host: torch.Tensor,
                                     paged_kv_last_page_len_host: torch.Tensor,
                                     paged_kv_indices_host: torch.Tensor, num_qo_heads: int,
                                     num_kv_heads: int, head_dim: int, page_size: int, device: torch.device,
-                                    target_workgroups: int = 0) -> torch.Tensor:
+                                    target_workgroups: int = 0, route_one_row_requests: bool = True) -> torch.Tensor:
         """begin_forward for callers that also have the step's other index arrays to upload
         (the forward context): metadata and plan travel in ONE pinned block and ONE upload
         kernel.  fill_metadata(view) writes the caller's meta_words int32 words (a multiple of
@@ -398,10 +416,11 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         h_qo = qo_indptr_host.to(torch.int32).contiguous()
         h_kv = paged_kv_indptr_host.to(torch.int32).contiguous()
         h_last = paged_kv_last_page_len_host.to(torch.int32).contiguous()
-        cap, kv_len = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices_host, paged_kv_indices_host)
+        cap = self._check_and_bound(h_qo, h_kv, h_last, paged_kv_indices_host, paged_kv_indices_host)
         block = staging.take(meta_words + max(cap, 4))
         fill_metadata(block.tensor[:meta_words])
-        words = self._plan_into(block.tensor[meta_words:], cap, h_qo, kv_len, target_workgroups)
+        words = self._plan_into(block.tensor[meta_words:], cap, h_qo, h_kv, h_last, target_workgroups,
+                                route_one_row_requests)
         dev = staging.to_device(block, meta_words + max(words, 4), device)
         batch = h_qo.shape[0] - 1
         used = int(h_kv[-1]) if batch > 0 else 0
@@ -414,19 +433,24 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         return dev[:meta_words]
 
     def forward(self, q: torch.Tensor, paged_kv_data: torch.Tensor, causal: bool = True,
-                sm_scale: Optional[float] = None, **_ignored) -> torch.Tensor:
+                sm_scale: Optional[float] = None, *, out: Optional[torch.Tensor] = None,
+                **_ignored) -> torch.Tensor:
+        """out: optional result tensor (contiguous, q's shape and dtype); every row is written."""
         if not self._planned:
             raise RuntimeError("prefill forward called before begin_forward")
         q = q.contiguous()
         if tuple(q.shape) != (self._nnz, self._hq, self._d):
             raise ValueError(f"q must be ({self._nnz}, {self._hq}, {self._d}), got {tuple(q.shape)}")
         self._check_pool(paged_kv_data, q.dtype)
-        out = torch.empty_like(q)
+        if out is None:
+            out = torch.empty_like(q)
+        elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+            raise ValueError("out must be contiguous and of q's shape and dtype")
         scale = 1.0 / math.sqrt(self._d) if sm_scale is None else sm_scale
-        rc = _lib.lib().dskv_prefill_attn(
+        rc = _lib.lib().dskv_mixed_attn(
             out.data_ptr(), q.data_ptr(), self._qo_indptr.data_ptr(), paged_kv_data.data_ptr(),
             self._indices.data_ptr(), self._indptr.data_ptr(), self._last.data_ptr(),
-            self._tiles.data_ptr(), self._n_tiles, self._n_splits, self._workspace.data_ptr(),
+            self._tiles.data_ptr(), ctypes.byref(self._info), self._workspace.data_ptr(),
             self._workspace.numel() * self._workspace.element_size(), self._batch, self._nnz, self._hq,
             self._hkv, self._d, self._p, scale, int(causal), _lib.dtype_code(q.dtype),
             _lib.current_stream())

@@ -109,3 +109,89 @@ def config5_context_lengths(seed: int = 5, batch: int = 128, median: int = 2048,
     here since the configuration leaves it open), clipped to [64, 32768]."""
     rng = np.random.default_rng(seed)
     return np.clip(np.exp(rng.normal(np.log(median), sigma, size=batch)), lo, hi).astype(np.int64)
+
+
+@dataclass
+class MixedWorkload:
+    """A step as the reference's decode-first join stage assembles it
+    (deserve_worker/engine/pipeline/stage/join.py:11-88): the running requests, one new
+    token each, then chunks of pending prompts up to the step's token budget."""
+    name: str
+    args: StageArgs
+    pool: PagePool
+    tables: PageTableAllocator
+    tasks: List[TaskData]
+    caches: List[PagedKVCache]
+    stage: KVStage
+    q: torch.Tensor     # (L, nnz, Hq, D): ragged, decode rows first
+    k: torch.Tensor     # (L, nnz, Hkv, D)
+    v: torch.Tensor
+    decode_ctx: np.ndarray     # tokens each decode request holds before the step
+    chunk_prior: np.ndarray    # tokens each chunked request holds before the step
+    chunk_lens: np.ndarray     # new tokens of each chunk
+
+    @property
+    def nnz(self) -> int:
+        return int(self.q.shape[1])
+
+    def kv_bytes_per_token(self) -> int:
+        n_kv = self.args.n_kv_heads or self.args.n_heads
+        return 2 * n_kv * (self.args.dim // self.args.n_heads) * self.pool.pages.element_size()
+
+    def decode_kv_tokens(self) -> int:
+        """kv tokens the decode rows attend over (each request's context plus its new token)."""
+        return int((self.decode_ctx + 1).sum())
+
+    def chunk_flops(self) -> int:
+        """4 * Hq * D * sum over chunks of (n * prior + n (n + 1) / 2)."""
+        hq, d = self.args.n_heads, self.args.dim // self.args.n_heads
+        return int(4 * hq * d * sum(int(n) * int(p) + int(n) * (int(n) + 1) // 2
+                                    for n, p in zip(self.chunk_lens, self.chunk_prior)))
+
+
+def make_mixed_workload(name: str, decode_ctx: Sequence[int], chunk_prior: Sequence[int],
+                        chunk_lens: Sequence[int], n_layers: int, n_heads: int, n_kv_heads: int = 8,
+                        head_dim: int = 128, page_size: int = 16, dtype: torch.dtype = torch.bfloat16,
+                        seed: int = 0, device: str = "cuda", spare_pages: int = 64) -> MixedWorkload:
+    """Decode requests that hold decode_ctx[b] tokens and get one more, followed by chunked
+    requests that hold chunk_prior[c] tokens and get chunk_lens[c] more.  Pool pages are
+    N(0, 1) and handed out in a seeded permutation; q / k / v of the step's tokens are N(0, 1)."""
+    dev = torch.device(device)
+    dctx = np.asarray(decode_ctx, dtype=np.int64)
+    prior, lens = np.asarray(chunk_prior, dtype=np.int64), np.asarray(chunk_lens, dtype=np.int64)
+    after = np.concatenate([dctx + 1, prior + lens])
+    need = int((-(-after // page_size)).sum()) + spare_pages
+    args = StageArgs(n_heads=n_heads, n_kv_heads=n_kv_heads, dim=n_heads * head_dim,
+                     page_size=page_size, n_layers=n_layers)
+    pool = GpuPagePool(n_layers, need, page_size, dev, dtype, n_kv_heads, head_dim)
+    fill_normal(pool.pages, seed + 1)
+    scatter_pool_order(pool, seed + 2)
+    max_ctx = int(-(-(after.max() + 1) // page_size) * page_size)
+    tables = PageTableAllocator(len(after), max_ctx, page_size, dev)
+    tasks, caches = [], []
+    for b, n in enumerate(dctx):
+        tasks.append(TaskData(f"{name}-d{b}", int(n), 1, 1, int(n), SamplingParams()))
+    for c, (p, n) in enumerate(zip(prior, lens)):
+        tasks.append(TaskData(f"{name}-c{c}", int(p), 1, int(n), int(p + n), SamplingParams()))
+    for t in tasks:
+        cache = PagedKVCache.empty(tables, pool)
+        cache.extend(t.start_pos)
+        caches.append(cache)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed + 3)
+    nnz = int(len(dctx) + lens.sum())
+    mk = lambda h: torch.randn((n_layers, nnz, h, head_dim), generator=g, device=dev,
+                               dtype=torch.float32).to(dtype)
+    return MixedWorkload(name, args, pool, tables, tasks, caches, KVStage(args, use_rope=False),
+                         mk(n_heads), mk(n_kv_heads), mk(n_kv_heads), dctx, prior, lens)
+
+
+def mixed_step_shape(seed: int, decode_rows: int = 75, token_budget: int = 512, lo: int = 256,
+                     hi: int = 4096):
+    """The step behind the reference's best published row (deserve_exp/exp_args.csv: microbatch
+    size 75; engine/pipeline/scheduler.py:74,85: 512 tokens per step): `decode_rows` running
+    requests with contexts seeded uniform in [lo, hi], and one chunk that fills the rest of
+    the token budget over a prior seeded uniform in [0, hi].  Returns (decode contexts,
+    [prior], [chunk length])."""
+    rng = np.random.default_rng(seed)
+    return rng.integers(lo, hi + 1, size=decode_rows), [int(rng.integers(0, hi + 1))], [token_budget - decode_rows]

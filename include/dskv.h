@@ -29,6 +29,13 @@ extern "C" {
 #define DSKV_BF16 2
 
 const char *dskv_last_error(void);
+/*
+ * DSKV_ABI_VERSION of the library that was loaded.  It changes whenever the signature of an
+ * exported function changes (the arguments are plain words and pointers: a caller built
+ * against another header would pass shifted arguments without any error), so a binding
+ * compares it with the value of the header it was written against before its first call.
+ */
+#define DSKV_ABI_VERSION 3
 int dskv_version(void);
 
 /*
@@ -227,6 +234,51 @@ int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const 
                       void *stream);
 
 /*
+ * Mixed batches.  The reference sends the WHOLE batch through its prefill wrapper as soon as
+ * one task of the step has more than one new token (engine/microbatch/processor.py:116-145),
+ * and its decode-first join stage (engine/pipeline/stage/join.py:11-88, 512-token budget)
+ * makes that the usual step: dozens of decode rows plus one chunk (benchmark/mixed.py:19-88
+ * times exactly this).  dskv_mixed_plan / dskv_mixed_attn are dskv_prefill_plan /
+ * dskv_prefill_attn for such batches: a request with ONE query row sees every kv token of
+ * its request with or without the causal mask, so it is a decode row - it is planned as
+ * split-KV decode items (dskv_decode_plan's work list, its K/V read once at the speed of
+ * memory) while the other requests are planned as query tiles; dskv_mixed_attn launches the
+ * decode pass over the one-row requests and the tile pass over the rest, and both write
+ * their rows of the same ragged `out`.  Routing needs a shape the 16-bit decode kernel
+ * takes (head_dim 128, group <= 16, power-of-two page) and route_one_row_requests != 0;
+ * otherwise, and for a batch without one-row requests, plan and result are those of
+ * dskv_prefill_plan / dskv_prefill_attn.  fp32 data is computed by the generic kernel,
+ * whatever the plan routed.
+ * The plan (at most dskv_mixed_plan_bound words; upload the first info->plan_words) holds
+ * the tile entries, then at word decode_plan_at the decode work list, at row_map_at the
+ * query row of every routed request and at tile_rows_at the rows the tiles cover.
+ * workspace: tile_workspace_bytes (partials of tile parts) + decode_workspace_bytes
+ * (partials of cut decode rows), 16-byte aligned.
+ */
+typedef struct dskv_mixed_plan {
+    int32_t n_tiles, n_splits;        /* tile entries (tiles x parts), parts per tile */
+    int32_t n_tile_rows;              /* query rows computed by the tile pass */
+    int32_t n_decode_rows;            /* one-row requests computed by the decode pass */
+    int32_t n_decode_items, n_decode_workgroups;
+    int64_t plan_words;
+    int64_t decode_plan_at, row_map_at, tile_rows_at;
+    int64_t tile_workspace_bytes, decode_workspace_bytes;
+} dskv_mixed_plan_t;
+int64_t dskv_mixed_plan_bound(int32_t batch, int64_t nnz, int64_t total_kv_tokens);
+int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_page_indptr_host,
+                    const int32_t *kv_last_page_len_host, int32_t batch, int32_t page_size,
+                    int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
+                    int32_t target_workgroups, int32_t route_one_row_requests,
+                    int32_t *plan_host, int64_t capacity_words, dskv_mixed_plan_t *info);
+int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indptr, const void *pages_layer,
+                    const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
+                    const int32_t *kv_last_page_len, const int32_t *plan_dev,
+                    const dskv_mixed_plan_t *info, void *workspace, int64_t workspace_bytes,
+                    int32_t batch, int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
+                    int32_t head_dim, int32_t page_size, float sm_scale, int32_t causal,
+                    int32_t dtype, void *stream);
+
+/*
  * Rotary embedding, adjacent-pair convention.  Replaces the call site
  * model/layer/attention.py:166-173 (flashinfer.apply_rope(q, k, indptr,
  * offsets, interleave=True, rope_theta=5e5)); maths as in
@@ -306,7 +358,8 @@ int dskv_swap_query(dskv_swap_t *handle, int32_t *done_out);
  * The two side streams of the engine (hipStream_t): [out] device-to-host, [in]
  * host-to-device.  Lets the bulk slice swap (dskv_swap_slice, the two streams of
  * kvcache/virtual.py:48-49) run on the engine's streams, so that a process holds three
- * streams - compute and these two - and not five.
+ * streams - compute and these two - and not five.  The handles stay valid until
+ * dskv_swap_destroy (after this call dskv_swap_bind_compute_stream no longer replaces them).
  */
 int dskv_swap_streams(dskv_swap_t *handle, void **out_stream, void **in_stream);
 /*
@@ -321,6 +374,9 @@ int dskv_swap_streams(dskv_swap_t *handle, void **out_stream, void **in_stream);
  * and each other, 0 if no such pair was found (the engine still works, without overlap).
  * No counterpart in the reference, whose two torch streams (kvcache/virtual.py:48-49)
  * are subject to the same sharing.
+ * Replacing a stream destroys it: handles obtained from dskv_swap_streams would dangle, so
+ * once that call has handed the streams out, binding is refused with DSKV_E_STATE.  Bind
+ * first (right after dskv_swap_create), then ask for the streams.
  */
 int dskv_swap_bind_compute_stream(dskv_swap_t *handle, void *compute_stream,
                                   int32_t *independent_out);

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol_and_binding_matches_header():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in dskv.h but not exported"
     assert sorted(_lib.EXPORTED_SYMBOLS) == declared
-    assert lib.dskv_version() == 1
+    assert lib.dskv_version() == _lib.ABI_VERSION == 3
 
 
 def test_argument_errors_return_negative_codes_without_a_gpu():
@@ -255,3 +255,91 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     no_keys = _prefill_plan(lib, qo2, np.array([4096, 0], np.int32), 32, 8, target=256)[1]
     none = no_keys[no_keys[:, 0] == 1]
     assert none[:, 2].tolist() == [0] * 8 and none[:, 3].tolist() == [0] * 7 + [0x7fffffff]
+
+
+def _mixed_plan(lib, qo_lens, kv_lens, P=16, hq=32, hkv=8, d=128, target=0, route=1, cap=None):
+    """Runs dskv_mixed_plan on requests given by (new tokens, kv tokens); returns (rc, info, plan)."""
+    qo = np.concatenate([[0], np.cumsum(qo_lens)]).astype(np.int32)
+    kv_lens = np.asarray(kv_lens, np.int64)
+    npages = -(-kv_lens // P)
+    indptr = np.concatenate([[0], np.cumsum(npages)]).astype(np.int32)
+    last = np.where(kv_lens > 0, (kv_lens - 1) % P + 1, 0).astype(np.int32)
+    cap = lib.dskv_mixed_plan_bound(len(qo_lens), int(qo[-1]), int(npages.sum()) * P) if cap is None else cap
+    plan = np.full(max(cap, 8), -7, np.int32)
+    info = _lib.MixedPlanInfo()
+    rc = lib.dskv_mixed_plan(qo.ctypes.data, indptr.ctypes.data, last.ctypes.data, len(qo_lens), P, hq, hkv, d,
+                             target, route, plan.ctypes.data, cap, ctypes.byref(info))
+    return rc, info, plan, qo, indptr
+
+
+def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest():
+    """The reference's mixed step (decode rows + one chunk through the prefill wrapper): every
+    one-row request with kv tokens appears in the decode work list exactly once over its whole
+    kv range, with its row of the ragged batch; every other row is covered by exactly one tile
+    (times the parts); the two row sets partition the batch."""
+    lib = _lib.lib()
+    rng = np.random.default_rng(5)
+    qo_lens = [1] * 20 + [300] + [1] * 10 + [0, 1, 2]
+    kv_lens = list(rng.integers(200, 4000, size=20)) + [2500] + list(rng.integers(1, 50, size=10)) + [40, 0, 2]
+    rc, info, plan, qo, indptr = _mixed_plan(lib, qo_lens, kv_lens)
+    assert rc == 0, _lib.last_error()
+    routed = [b for b in range(len(qo_lens)) if qo_lens[b] == 1 and kv_lens[b] > 0]
+    assert info.n_decode_rows == len(routed) == 30 and info.n_tile_rows == 300 + 1 + 2
+    assert info.n_decode_rows + info.n_tile_rows == int(qo[-1])
+    # tiles: only requests 20 (300 rows), 32 (one row without kv tokens) and 33 (two rows)
+    tiles = plan[: 5 * info.n_tiles].reshape(-1, 5)
+    assert sorted(set(tiles[:, 0].tolist())) == [20, 32, 33]
+    assert info.n_tiles == (5 + 1 + 1) * info.n_splits
+    assert info.decode_plan_at % 4 == 0 and info.decode_plan_at >= 5 * info.n_tiles
+    # the decode work list has dskv_decode_plan's layout; its items name ragged rows
+    dp = plan[info.decode_plan_at:]
+    n_items, wgs, n_slots, batch = dp[:4].tolist()
+    assert (n_items, wgs, batch) == (info.n_decode_items, info.n_decode_workgroups, info.n_decode_rows)
+    items = dp[4 + wgs + 1 + 2 * batch: 4 + wgs + 1 + 2 * batch + 8 * n_items].reshape(-1, 8)
+    assert info.row_map_at == info.decode_plan_at + 4 + wgs + 1 + 2 * batch + 8 * n_items
+    row_map = plan[info.row_map_at: info.row_map_at + batch]
+    assert row_map.tolist() == [int(qo[b]) for b in routed]
+    for i, b in enumerate(routed):
+        mine = items[items[:, 0] == qo[b]]
+        spans = sorted((t0, t1) for _, t0, t1, *_ in mine.tolist())
+        assert spans[0][0] == 0 and spans[-1][1] == kv_lens[b]
+        assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))
+        assert (mine[:, 4] == indptr[b]).all()                     # the request's block table
+        assert mine[mine[:, 2] == kv_lens[b]][:, 5].tolist() == [1]
+    tile_rows = plan[info.tile_rows_at: info.tile_rows_at + info.n_tile_rows]
+    assert info.plan_words == info.tile_rows_at + info.n_tile_rows
+    assert sorted(tile_rows.tolist() + row_map.tolist()) == list(range(int(qo[-1])))
+    assert info.decode_workspace_bytes == n_slots * 32 * 130 * 4
+    assert info.tile_workspace_bytes % 256 == 0
+    assert info.tile_workspace_bytes >= (info.n_splits > 1) * int(qo[-1]) * info.n_splits * 32 * 130 * 4
+
+
+def test_mixed_plan_without_routing_is_the_prefill_plan():
+    lib = _lib.lib()
+    qo_lens, kv_lens = [1, 1, 200, 1], [700, 33, 900, 16]
+    qo = np.concatenate([[0], np.cumsum(qo_lens)]).astype(np.int32)
+    _, want, splits, _, ws = _prefill_plan(lib, qo, np.array(kv_lens, np.int32), 32, 8)
+    for kwargs in (dict(route=0), dict(d=64), dict(hq=64, hkv=2), dict(P=12)):
+        if kwargs.get("d") == 64 or kwargs.get("hq") == 64:
+            _, want_k, splits_k, _, ws_k = _prefill_plan(lib, qo, np.array(kv_lens, np.int32), kwargs.get("hq", 32),
+                                                         kwargs.get("hkv", 8), head_dim=kwargs.get("d", 128))
+        else:
+            want_k, splits_k, ws_k = want, splits, ws
+        rc, info, plan, _, _ = _mixed_plan(lib, qo_lens, kv_lens, **kwargs)
+        assert rc == 0, (kwargs, _lib.last_error())
+        assert info.n_decode_rows == 0 and info.n_decode_items == 0 and info.decode_workspace_bytes == 0
+        assert info.n_tile_rows == 203 and info.n_splits == splits_k
+        assert plan[: info.plan_words].tolist() == want_k.reshape(-1).tolist()
+        assert info.tile_workspace_bytes == -(-ws_k // 256) * 256
+    # a batch of decode rows only (the reference's benchmark/mixed.py without a chunk): no tiles
+    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 1], [700, 33, 16])
+    assert rc == 0 and info.n_tiles == 0 and info.n_tile_rows == 0 and info.n_decode_rows == 3
+    assert info.decode_plan_at == 0
+    # refusals
+    assert _mixed_plan(lib, [1, 5], [700, 33], cap=6)[0] == -2
+    assert _mixed_plan(lib, [1, 200], [700, 900], cap=5 * 4 + 8)[0] == -2
+    assert _mixed_plan(lib, [1, 5], [700, 33], hq=30)[0] == -1
+    assert lib.dskv_mixed_plan(None, None, None, 0, 16, 32, 8, 128, 0, 1, None, 0, None) == -1
+    info = _lib.MixedPlanInfo()
+    assert lib.dskv_mixed_plan(None, None, None, 0, 16, 32, 8, 128, 0, 1, None, 0, ctypes.byref(info)) == 0
+    assert lib.dskv_mixed_attn(16, 16, 16, 16, 16, 16, 16, 16, None, None, 0, 1, 1, 32, 8, 128, 16, 0.1, 1, 2, None) == -1

@@ -222,9 +222,11 @@ def test_config3_microbatch_exchange_round_trip_full_size():
     eng.close()
 
 
-def test_config4_chunked_prefill_full_batch_four_layers():
+def test_config4_chunked_prefill_full_batch_all_layers():
     """16 sequences append a 512-token chunk behind a prior of U[0, 8192] tokens that ends
-    mid-page (offset U[0, 15]), then attend causally over prior + chunk."""
+    mid-page (offset U[0, 15]), then attend causally over prior + chunk: all 16 layers of
+    the stage; append read-back and checksum on every layer, sampled rows against the
+    oracle on four of them."""
     from deserve_amd.kvcache.paged.kvcache import PagedKVCache
     from deserve_amd.kvcache.paged.page_pool import GpuPagePool
     from deserve_amd.kvcache.paged.page_table import PageTableAllocator
@@ -234,7 +236,7 @@ def test_config4_chunked_prefill_full_batch_four_layers():
     from deserve_amd.task import SamplingParams, TaskData
 
     _announce("config4")
-    L, P, Hq, Hkv, D, B, n = 4, 16, 32, 8, 128, 16, 512
+    L, P, Hq, Hkv, D, B, n = 16, 16, 32, 8, 128, 16, 512
     rng = np.random.default_rng(4)
     prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
     prior[0], prior[1] = 0, 8192 + 15                               # extremes: pure prompt, longest
@@ -280,7 +282,8 @@ def test_config4_chunked_prefill_full_batch_four_layers():
     # the longest prior (requests 0 and 1), a row that ends on a page boundary, and seeded ones
     # over all requests; every row against its own output scale.
     worst = 0.0
-    for layer in range(L):
+    for layer in (0, 5, 10, 15):
+        assert np.isfinite(outs[layer].float().sum().item())
         picks = [(0, 0), (0, n - 1), (1, 0), (1, n - 1), (2, int((-prior[2] - 1) % P))]
         picks += [(int(rng.integers(0, B)), int(rng.integers(0, n))) for _ in range(11)]
         reqs = sorted({b for b, _ in picks})
@@ -370,9 +373,10 @@ def test_config5_fragmented_pool_swap_in_then_decode():
     wl = DecodeWorkload("cfg5", args, pool, rows, tasks, caches, KVStage(args, use_rope=False),
                         mk(Hq), mk(Hkv), mk(Hkv), ctx_lens)
     wrapper, _ = get_wrappers(DEV)
-    # 16 requests against the oracle: the longest (32 k tokens, cut into dozens of parts), the
-    # shortest, four of the swapped ones and seeded others; one layer with the append inside
-    # the attention launch (what the bench times) and, a step later, one with the two calls
+    # One layer with the append inside the attention launch (what the bench times): all 128
+    # requests against the oracle.  A step later, one layer with the two calls: 16 requests -
+    # the longest (32 k tokens, cut into dozens of parts), the shortest, four of the swapped
+    # ones and seeded others
     sample = [int(np.argmax(ctx_lens)), int(np.argmin(ctx_lens))] + swapped[:2] + swapped[-2:]
     sample += [int(b) for b in rng.permutation(B) if int(b) not in sample][: 16 - len(sample)]
     assert ctx_lens.max() == 32768
@@ -381,6 +385,8 @@ def test_config5_fragmented_pool_swap_in_then_decode():
         ctx, outs, (n_items, _) = _decode_step(wl, wrapper, [layer], fused=fused)
         assert n_items > B
         _check_append(wl, ctx, layer, before, old)
+        if fused:
+            sample = list(range(B))       # the benched form: every request of the layer
         want = _oracle_rows(wl, ctx, layer, sample)
         got = outs[layer].float().cpu().numpy()
         assert np.isfinite(got).all()
@@ -389,3 +395,60 @@ def test_config5_fragmented_pool_swap_in_then_decode():
         assert err <= 2e-2, (layer, fused)
         for t in tasks:
             t.step()
+
+
+def test_mixed_step_full_size_through_batch_prefill():
+    """The reference's usual step in its decode-first aggregated mode: 75 running requests
+    (contexts U[256, 4096], one new token each) and one chunk that fills the 512-token budget
+    over a prior of U[0, 4096] tokens, all through BatchPrefill (engine/microbatch/processor.py:
+    116-145) at the Llama-3-8B stage shape and again at the 70B shape.  The decode rows take
+    the split-KV decode kernel, the chunk the query tiles.  EVERY row of the ragged output of
+    two layers against the C oracle, each row against its own scale; the appended rows read
+    back bit for bit; the layer's checksum moves by exactly the appended rows."""
+    from deserve_amd.execution.exec import BatchPrefill, get_wrappers
+    from deserve_amd.synthetic import make_mixed_workload, mixed_step_shape
+
+    for tag, L, Hq in (("8B", 3, 32), ("70B", 2, 64)):
+        _announce("mixed step", tag)
+        P, Hkv, D = 16, 8, 128
+        dctx, prior, lens = mixed_step_shape(11)
+        prior[0] = max(prior[0], 1500)                                  # the chunk is planned in parts
+        wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=11)
+        nnz, n_dec = wl.nnz, len(dctx)
+        assert nnz == 512
+        before = [_checksum(wl.pool.pages[l]) for l in range(L)]
+        step = BatchPrefill((wl.q, wl.k, wl.v), wl.stage, wl.tasks, wl.caches)
+        step.prepare()
+        ctx = step.prefill_ctx
+        _, w = get_wrappers(DEV)
+        assert w._n_decode_rows == n_dec and w._info.n_tile_rows == nnz - n_dec
+        assert w._n_splits > 1                                          # 7 tiles x 8 heads: cut into parts
+        indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
+        last, qo = ctx.host["kv_last_page_lens"].numpy(), ctx.host["indptr"].numpy()
+        start = np.array([t.start_pos for t in wl.tasks])
+        n_new = np.diff(qo)
+        pos = np.concatenate([np.arange(s, s + n) for s, n in zip(start, n_new)])
+        req = np.repeat(np.arange(len(wl.tasks)), n_new)
+        page = torch.from_numpy(ids_all[indptr[req] + pos // P].astype(np.int64)).to(DEV)
+        slot = torch.from_numpy((pos % P).astype(np.int64)).to(DEV)
+        old = [_checksum(wl.pool.pages[l][page, :, slot]) for l in range(L)]
+        result = step.step(ignore_eos=True).all_xs               # the stage's output (no sampling here)
+        torch.cuda.synchronize()
+        assert result.shape == (L, nnz, Hq * D)
+        for l in range(L):
+            got_rows = wl.pool.pages[l][page, :, slot]
+            assert torch.equal(got_rows[:, 0].view(torch.int16), wl.k[l].view(torch.int16))
+            assert torch.equal(got_rows[:, 1].view(torch.int16), wl.v[l].view(torch.int16))
+            assert _checksum(wl.pool.pages[l]) == before[l] - old[l] + _checksum(wl.k[l]) + _checksum(wl.v[l])
+        for l in (0, L - 1):
+            pages = _bits(wl.pool.pages[l].index_select(0, torch.from_numpy(ids_all.astype(np.int64)).to(DEV)))
+            want = c_oracle.prefill_attn(_bits(wl.q[l]), qo, pages, np.arange(len(ids_all), dtype=np.int32),
+                                         indptr, last, "bf16", causal=True)
+            got = result[l].view(nnz, Hq, D).float().cpu().numpy()
+            assert np.isfinite(got).all()
+            err_dec = max_rel_err_per_request(got[:n_dec], want[:n_dec])
+            err_chunk = max_rel_err_per_request(got[n_dec:], want[n_dec:])
+            _announce("mixed", tag, "layer", l, "worst decode row", err_dec, "worst chunk row", err_chunk)
+            assert err_dec <= 2e-2 and err_chunk <= 2e-2, (tag, l)
+        del wl, result, step
+        torch.cuda.empty_cache()

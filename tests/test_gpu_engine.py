@@ -473,3 +473,53 @@ def test_staged_uploads_are_exact_and_blocks_wait_for_their_readers():
         assert np.array_equal(o.cpu().numpy(), r)
     with pytest.raises(ValueError):
         staging.upload(staging.take(4), torch.zeros(2, dtype=torch.int32, device=dev), 4)
+
+
+def test_step_request_with_device_tensors_crosses_the_stage_hop_bit_for_bit():
+    """The stage hop (deserve_worker/request.py:199-210, engine/pipeline/processor.py:224): a
+    StepRequest whose activations live on the GPU goes through into_safetensors -> dumps ->
+    loads -> from_safetensors back onto the device.  The tensor that arrives has the bits of
+    the one that left, the metadata is equal, and a decode step driven by what arrived gives
+    the outputs and the pages of the same step driven by the original."""
+    from deserve_amd import serde
+    from deserve_amd.engine.pipeline.processor import StepRequest
+    from deserve_amd.execution.exec import BatchDecode
+    from deserve_amd.stage import PackedKVStage
+    from deserve_amd.synthetic import make_decode_workload
+    from deserve_amd.task import SamplingParams
+
+    ctx_lens = [700, 33, 16, 1, 2049, 255, 4000, 90]
+    sides = [make_decode_workload("hop", ctx_lens, L, HQ, HKV, D, P, torch.bfloat16, headroom_tokens=8, seed=21)
+             for _ in range(2)]
+    a, b = sides
+    assert torch.equal(a.pool.pages.view(torch.int16), b.pool.pages.view(torch.int16))
+    # one tensor per token, as the scheduler's queues carry it: (B, L, Hq + 2 Hkv, D)
+    xs = torch.cat([a.q, a.k, a.v], dim=2).permute(1, 0, 2, 3).contiguous()
+    ids = [t.task_id for t in a.tasks]
+    req = StepRequest(3, xs, exec_task_ids=list(ids), exec_seqlens=[1] * len(ids), cancel_task_ids=["gone"],
+                      offload_task_ids=[ids[1]], reload_task_ids=[],
+                      init_tasks={ids[0]: (700, SamplingParams(temperature=0.5, max_new_tokens=7))})
+    assert req.xs.is_cuda
+    wire = serde.dumps(*req.into_safetensors())
+    assert isinstance(wire, bytes) and len(wire) > req.get_tensors_size()
+    back = StepRequest.from_safetensors(*serde.loads(wire), device=DEV)
+    assert back.xs.is_cuda and back.xs.dtype == xs.dtype and back.xs.shape == xs.shape
+    assert torch.equal(back.xs.view(torch.int16), xs.view(torch.int16))
+    for name in ("microbatch_id", "exec_task_ids", "exec_seqlens", "cancel_task_ids", "offload_task_ids",
+                 "reload_task_ids"):
+        assert getattr(back, name) == getattr(req, name), name
+    assert back.init_tasks[ids[0]][0] == 700 and back.init_tasks[ids[0]][1].model_dump() == \
+        req.init_tasks[ids[0]][1].model_dump()
+    outs = []
+    for side, x in ((a, req.xs), (b, back.xs)):
+        step = BatchDecode(x, PackedKVStage(side.args, use_rope=True), side.tasks, side.caches)
+        step.prepare()
+        outs.append(step.step(ignore_eos=True).all_xs)
+    torch.cuda.synchronize()
+    assert outs[0].shape == (L, len(ids), HQ * D)
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(a.pool.pages.view(torch.int16), b.pool.pages.view(torch.int16))
+    # an empty request keeps the reference's quirk on the way (a one-element stand-in) and comes back empty
+    empty = StepRequest.from_safetensors(*serde.loads(serde.dumps(*StepRequest.empty(0, torch.bfloat16, DEV).into_safetensors())),
+                                         device=DEV)
+    assert empty.is_empty() and empty.xs.is_cuda and empty.xs.dtype == torch.bfloat16

@@ -428,6 +428,30 @@ def test_decode_with_rope_inside_equals_rope_append_then_decode(case):
     w.end_forward()
 
 
+def test_fused_append_refuses_a_request_without_pages_and_touches_nothing():
+    """kv lengths [0, 40, 3]: request 0 owns no page, so its token has no slot.  The call is
+    refused on the host; pages and output stay as they were.  The same plan without the
+    append still runs (request 0 yields zeros)."""
+    from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
+
+    _announce("decode fused append, empty request")
+    sc = make_scenario(914, kv_lens=[0, 40, 3], qo_lens=[1, 1, 1], dtype="bf16")
+    w = BatchDecodeWithPagedKVCacheWrapper(torch.empty(8 << 20, dtype=torch.uint8, device="cuda"))
+    w.begin_forward(_dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                    _dev_i32(sc.kv_last_page_lens), sc.Hq, sc.Hkv, sc.D, sc.P)
+    q, k, v, pages = (to_torch(x, "bf16") for x in (sc.q, sc.k, sc.v, sc.pages))
+    out = torch.full_like(q, 7.0)
+    with pytest.raises(ValueError, match="have no page"):
+        w.forward(q, pages, k_append=k, v_append=v, out=out)
+    torch.cuda.synchronize()
+    assert _same_bits(from_torch(pages, "bf16"), sc.pages) and bool((out == 7.0).all())
+    got = w.forward(q, pages).float().cpu().numpy()
+    want = c_oracle.decode_attn(sc.q, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                sc.kv_last_page_lens, "bf16")
+    assert not got[0].any() and max_rel_err_per_request(got[1:], want[1:]) <= 2e-2
+    w.end_forward()
+
+
 def test_fused_append_is_refused_outside_the_mfma_shapes():
     from deserve_amd.paged_ops import BatchDecodeWithPagedKVCacheWrapper
 
@@ -443,6 +467,56 @@ def test_fused_append_is_refused_outside_the_mfma_shapes():
         w.forward(to_torch(sc.q, "f32"), pages, k_append=to_torch(sc.k, "f32"), v_append=to_torch(sc.v, "f32"))
     torch.cuda.synchronize()
     assert _same_bits(from_torch(pages, "f32"), before)
+
+
+# ------------------------------------------------------------------ mixed batches
+MIXED_CASES = [
+    # (name, kv_lens, qo_lens, P, Hq, Hkv, dtype, target_workgroups, rows routed to the decode kernel)
+    ("decode_rows_and_chunk", [700, 33, 16, 900, 2049, 5], [1, 1, 1, 120, 1, 5], 16, 32, 8, "bf16", 0, 4),
+    ("cut_rows", [4096, 3000, 257, 1500, 700], [1, 1, 1, 64, 1], 16, 32, 8, "bf16", 64, 4),
+    ("chunk_first_and_last", [600, 40, 77, 1], [200, 1, 1, 1], 16, 32, 8, "bf16", 0, 3),
+    ("group8_f16_page8", [3000, 2049, 64, 9], [65, 1, 1, 1], 8, 64, 8, "f16", 0, 3),
+    ("only_decode_rows", [700, 33, 16, 1], [1, 1, 1, 1], 16, 32, 8, "bf16", 0, 4),
+    ("row_without_kv", [0, 40, 300], [1, 1, 8], 16, 32, 8, "bf16", 0, 1),
+    ("page4", [100, 37, 64], [1, 20, 1], 4, 32, 8, "f16", 0, 2),
+    ("page2_mha", [50, 37, 64], [1, 20, 1], 2, 8, 8, "bf16", 0, 2),
+    ("f32_generic_kernel", [100, 37, 64], [1, 20, 1], 16, 32, 8, "f32", 0, 2),
+    ("group32_stays_tiled", [100, 37, 64], [1, 20, 1], 16, 32, 1, "bf16", 0, 0),
+    ("many_rows", [17 * i % 900 + 1 for i in range(75)] + [2500], [1] * 75 + [437], 16, 32, 8, "bf16", 0, 75),
+]
+
+
+@pytest.mark.parametrize("case", MIXED_CASES, ids=[c[0] for c in MIXED_CASES])
+def test_mixed_batch_routes_one_row_requests_to_the_decode_kernel(case):
+    """The reference's mixed step sends decode rows and a chunk through the prefill wrapper
+    together (engine/microbatch/processor.py:116-145).  The wrapper computes the one-row
+    requests with the split-KV decode kernel and the rest with query tiles; every row of
+    the ragged output - written into a NaN-filled tensor - matches the oracle's prefill
+    attention, with and without the mask, as it does with the routing switched off."""
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+
+    name, kv, qo, P, Hq, Hkv, dtype, target, n_routed = case
+    _announce("mixed", name, P, Hq, Hkv, dtype, target)
+    sc = make_scenario(43, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(96 << 20, dtype=torch.uint8, device="cuda"))
+    q, pages = to_torch(sc.q, dtype), to_torch(sc.pages, dtype)
+    for route in (True, False):
+        w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                        _dev_i32(sc.kv_last_page_lens), Hq, Hkv, 128, P, target_workgroups=target,
+                        route_one_row_requests=route)
+        assert w._n_decode_rows == (n_routed if route else 0)
+        if name == "cut_rows" and route:
+            assert w._info.n_decode_items > w._n_decode_rows          # rows cut across workgroups: merged
+        for causal in (True, False):
+            out = torch.full_like(q, float("nan"))
+            assert w.forward(q, pages, causal=causal, out=out) is out
+            torch.cuda.synchronize()
+            got = out.float().cpu().numpy()
+            want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
+                                         sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
+            assert np.isfinite(got).all(), (name, route, causal)
+            assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (name, route, causal)
+        w.end_forward()
 
 
 def test_prefill_with_one_query_equals_decode():

@@ -56,6 +56,31 @@ def test_forward_refuses_a_pool_that_lacks_a_named_page_or_has_another_shape():
         w._check_pool(torch.empty((41, 2, 16, 8, 256), dtype=torch.bfloat16)[..., ::2], torch.bfloat16)
 
 
+def test_fused_append_refuses_a_plan_with_a_request_that_owns_no_page():
+    """forward(k_append=) writes the step's token into the page slot the block table names
+    for it (model/layer/attention.py:175-185): a request without a page has no such slot, and
+    the refusal comes from the host, before anything is launched."""
+    from deserve_amd import _lib
+
+    w = _decode()
+    w._shape_args(32, 8, 128, 16)
+    h_indptr, h_last = _i32([0, 0, 3, 4]), _i32([16, 8, 3])
+    w._check_block_tables(h_indptr, _i32([1, 2, 3, 0]), None, h_last)
+    cap = int(_lib.lib().dskv_decode_plan_bound(3, 4 * 16))
+    w._plan_into(torch.zeros(cap, dtype=torch.int32), cap, h_indptr, h_last, 0)
+    assert w._empty_requests == [0]
+    w._planned = True
+    q = torch.zeros((3, 32, 128), dtype=torch.bfloat16)
+    k = torch.zeros((3, 8, 128), dtype=torch.bfloat16)
+    pages = torch.zeros((4, 2, 16, 8, 128), dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="\\[0\\] have no page"):
+        w.forward(q, pages, k_append=k, v_append=k)
+    assert not pages.any()
+    # a plan whose requests all own a page passes this check
+    w._plan_into(torch.zeros(cap, dtype=torch.int32), cap, _i32([0, 1, 3, 4]), h_last, 0)
+    assert w._empty_requests == []
+
+
 def test_prefill_begin_forward_refuses_bad_block_tables():
     w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(16, dtype=torch.uint8))
     shape = dict(num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16)
