@@ -60,7 +60,9 @@ def parse_args():
                          "output on before it starts the next but one); 0 = no limit")
     ap.add_argument("--no-rope-step", action="store_true", help="skip the extra steps with rotation")
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
-    ap.add_argument("--section", choices=["swap", "fragmented", "prefill"], default=None,
+    ap.add_argument("--no-mixed", action="store_true", help="skip the mixed decode + chunk section")
+    ap.add_argument("--no-page8", action="store_true", help="skip configuration 2 on 8-token pages")
+    ap.add_argument("--section", choices=["swap", "fragmented", "prefill", "mixed", "mfma-ceiling"], default=None,
                     help="(internal) run only this host-link section and print its JSON object")
     ap.add_argument("--page-size", type=int, default=16,
                     help="tokens per page of the benched pool (BASELINE's configurations use 16; the "
@@ -72,6 +74,8 @@ def parse_args():
                     help="with --section prefill: only configuration 4's launches on its own data "
                          "(20 appends, 20 attention launches), for profiler runs whose per-kernel "
                          "averages must not mix in the zero-data and one-chunk measurements")
+    ap.add_argument("--mixed-shapes", default="8B,70B",
+                    help="with --section mixed: which stage shapes to run (8B, 70B)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -198,7 +202,7 @@ def cpu_reference_config1(seed: int):
     err = max(float(np.abs(got[b] - want[b]).max() / np.abs(want[b]).max()) for b in range(B))
     same_pages = bool(torch.equal(d_pages.cpu(), pages[0]))
     return {"value": round(nbytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": threads,
-            "kind": "reference-restatement", "config": "configs[0]",
+            "kind": "port", "config": "configs[0]",
             "sample": f"BASELINE.json configs[0] exactly: 1 layer fp32, 8 x 512 tokens after the append, 256-page "
                       f"pool in a seeded permutation; torch CPU ({threads} threads): index-assign append, "
                       f"pages[layer, table] gather, repeat_kv + softmax(scores.float()) matmuls; median of 30 "
@@ -433,6 +437,18 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
                               c.kv_page_indptr, c.kv_last_page_lens)
 
     append_us = median_us(append)
+    # the chunk's rotation: apply_rope alone, and rotation + append in one pass (what a layer
+    # runs in front of the attention: q rotated out of place, rotated k and v into their slots)
+    from deserve_amd.paged_ops import apply_rope, rope_append_paged_kv_cache
+    offsets = torch.from_numpy(prior.astype(np.int32)).to(dev)
+    rope_us = median_us(lambda layer: apply_rope(q[layer], k[layer], c.indptr, offsets, interleave=True,
+                                                 rope_theta=5e5))
+    rope_append_us = median_us(lambda layer: rope_append_paged_kv_cache(
+        q[layer], k[layer], v[layer], c.indptr, offsets, pool.pages[layer], c.kv_page_indices,
+        c.kv_page_indptr, c.kv_last_page_lens, rope_theta=5e5))
+    append(0), append(1), append(2), append(3)          # the unrotated rows again, as the attention figures assume
+    rope_bytes = 2 * B * n * (Hq + Hkv) * D * 2
+    rope_append_bytes = 2 * B * n * (Hq + 2 * Hkv) * D * 2
     attn_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
     result = {"workload": "BASELINE.json configs[3]: bf16, GQA 32q/8kv, page 16, 16 sequences x 512-token "
                           "chunk appended at offsets U[0,15], attention over prior U[0,8192]; per layer",
@@ -442,7 +458,14 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
               "attention_us_per_layer": round(attn_us, 1),
               "attention_TFLOPs": round(flops / attn_us / 1e6, 1),
               "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
-              "flops_per_layer": flops}
+              "flops_per_layer": flops,
+              "rope": {"workload": f"the chunk's {B * n} tokens x ({Hq} q + {Hkv} kv heads), positions from the priors",
+                       "apply_rope_us_per_layer": round(rope_us, 1),
+                       "apply_rope_bytes": rope_bytes,
+                       "apply_rope_frac_of_hbm_peak": round(rope_bytes / rope_us / 1e3 / HBM_PEAK_GBPS, 4),
+                       "rope_append_us_per_layer": round(rope_append_us, 1),
+                       "rope_append_bytes": rope_append_bytes,
+                       "rope_append_frac_of_hbm_peak": round(rope_append_bytes / rope_append_us / 1e3 / HBM_PEAK_GBPS, 4)}}
     if not extras:
         w.end_forward()
         return result
@@ -455,10 +478,190 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
     attn_zero_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
     w.end_forward()
     one_chunk = one_chunk_measure(gen)
-    result.update({"attention_us_per_layer_zero_data": round(attn_zero_us, 1),
+    ceiling = mfma_ceiling_section(seed)
+    measured_peak = ceiling["levels"]["mfma_only"]["normal"]
+    result.update({"mfma_ceiling": ceiling,
+                   "frac_of_measured_mfma_ceiling": round(result["attention_TFLOPs"] / measured_peak, 4),
+                   "attention_us_per_layer_zero_data": round(attn_zero_us, 1),
                    "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
                    "one_512_token_chunk_over_4096": one_chunk})
     return result
+
+
+def mfma_ceiling_section(seed: int, levels=(0, 1, 2), fills=("normal", "constant")):
+    """What the matrix pipeline sustains on this box, measured with the calibration loop of
+    deserve_amd/csrc/calib/mfma_ceiling.hip (16 v_mfma_f32_32x32x16_bf16 per iteration and
+    wave, 1024 workgroups of 8 waves): level 0 the MFMAs alone, level 1 with the LDS operand
+    reads of a 32-token attention block, level 2 with its softmax as well - on N(0, 1)
+    operands and on constant ones.  The prefill kernel's rate is read against level 0 on
+    N(0, 1) data (`frac_of_measured_mfma_ceiling`) beside the published peak."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(ROOT, "deserve_amd", "libdskv_calib.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it (python -c 'import __graft_entry__ as g; g.build()')")
+    lib = ctypes.CDLL(path)
+    lib.dskv_calib_mfma_loop.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+    lib.dskv_calib_mfma_loop_flops.restype = ctypes.c_double
+    lib.dskv_calib_mfma_loop_flops.argtypes = [ctypes.c_int, ctypes.c_int]
+    dev = torch.device("cuda")
+    wgs, iters = 1024, 1536
+    g = torch.Generator(device=dev).manual_seed(seed + 70)
+    data = {"normal": torch.randn(512 * 128, generator=g, device=dev).to(torch.bfloat16),
+            "constant": torch.full((512 * 128,), 1.0, device=dev, dtype=torch.bfloat16)}
+    sink = torch.empty(wgs * 512, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    names = {0: "mfma_only", 1: "plus_lds_operand_reads", 2: "plus_lds_operand_reads_and_softmax"}
+    out = {"loop": "16 x v_mfma_f32_32x32x16_bf16 per wave and iteration, 8 waves per workgroup, "
+                   f"{wgs} workgroups x {iters} iterations; TFLOP/s", "levels": {}}
+    flops = lib.dskv_calib_mfma_loop_flops(wgs, iters)
+    for level in levels:
+        row = {}
+        for fill in fills:
+            ts = []
+            for rep_ in range(4):
+                a_, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a_.record()
+                rc = lib.dskv_calib_mfma_loop(data[fill].data_ptr(), sink.data_ptr(), level, wgs, iters,
+                                              0.1275, stream)
+                b_.record()
+                if rc != 0:
+                    raise RuntimeError(f"dskv_calib_mfma_loop failed with code {rc}")
+                torch.cuda.synchronize()
+                ts.append(a_.elapsed_time(b_))
+            ms = sorted(ts[1:])[1]
+            row[fill] = round(flops / ms / 1e9, 1)
+        out["levels"][names[level]] = row
+    out["frac_of_published_peak_mfma_only_normal_data"] = round(
+        out["levels"]["mfma_only"]["normal"] / MFMA_PEAK_BF16_TFLOPS, 4) if 0 in levels and "normal" in fills else None
+    return out
+
+
+def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
+    """The reference's usual step in its decode-first aggregated mode (engine/pipeline/stage/
+    join.py:11-88, 512-token budget; deserve_exp/exp_args.csv: microbatch size 75): 75 running
+    requests with contexts U[256, 4096], one new token each, plus one chunk that fills the
+    rest of the budget (437 tokens) over a prior U[0, 4096] - all sent through the prefill
+    wrapper, as engine/microbatch/processor.py:116-145 does whenever one task has more than one
+    token.  Per layer, on the launch stream: the append of the step's 512 tokens and the
+    attention call, with the one-row requests routed to the split-KV decode kernel and
+    without; the decode rows alone and the chunk alone give the two roofline fractions."""
+    import numpy as np
+    import torch
+
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.model.context.flash import FlashPrefillCtx
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper, append_paged_kv_cache
+    from deserve_amd.synthetic import make_mixed_workload, mixed_step_shape
+
+    dev = torch.device("cuda")
+    P, Hkv, D = 16, 8, 128
+    out = {"workload": "75 decode rows, ctx U[256,4096], + one 437-token chunk over a prior U[0,4096] (512-token "
+                       "step budget), bf16, page 16, through the prefill wrapper; per layer"}
+    for tag in shapes:
+        L, Hq = {"8B": (16, 32), "70B": (10, 64)}[tag]
+        dctx, prior, lens = mixed_step_shape(seed + 60)
+        wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=seed + 61)
+        n_dec, nnz = len(dctx), wl.nnz
+        tok_bytes = wl.kv_bytes_per_token()
+        _, w = get_wrappers(dev)
+        settle_heap()
+
+        def plan(tasks, caches, route=True):
+            return FlashPrefillCtx.init_and_plan(tasks, caches, w, Hq, Hkv, D, P) if route else None
+
+        def median_us(fn, layers=L):
+            evs = []
+            for _ in range(reps):
+                for layer in range(layers):
+                    s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    s_.record()
+                    fn(layer)
+                    e_.record()
+                    evs.append((s_, e_))
+            torch.cuda.synchronize()
+            ts = sorted(a.elapsed_time(b) for a, b in evs[L:])          # the first pass warms up
+            return ts[len(ts) // 2] * 1e3
+
+        c = FlashPrefillCtx.init_and_plan(wl.tasks, wl.caches, w, Hq, Hkv, D, P)
+        routed_rows, parts = w._n_decode_rows, w._n_splits
+        n_pages = int(c.host["kv_page_indptr"][-1])
+        append_us = median_us(lambda l: append_paged_kv_cache(wl.k[l], wl.v[l], c.indptr, wl.pool.pages[l],
+                                                              c.kv_page_indices, c.kv_page_indptr,
+                                                              c.kv_last_page_lens))
+        mixed_us = median_us(lambda l: w.forward(wl.q[l], wl.pool.pages[l], causal=True))
+        w.end_forward()
+        # the whole step as the engine runs it: plan + upload, then L x (append + attention)
+        def step():
+            cc = FlashPrefillCtx.init_and_plan(wl.tasks, wl.caches, w, Hq, Hkv, D, P)
+            for l in range(L):
+                append_paged_kv_cache(wl.k[l], wl.v[l], cc.indptr, wl.pool.pages[l], cc.kv_page_indices,
+                                      cc.kv_page_indptr, cc.kv_last_page_lens)
+                w.forward(wl.q[l], wl.pool.pages[l], causal=True)
+            w.end_forward()
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        step_ms = (time.perf_counter() - t0) / 10 * 1e3
+        # the same batch with every request on the tile path (a one-row request = one live
+        # row of a 64-row tile): what the step cost before the routing
+        w2 = BatchPrefillWithPagedKVCacheWrapper(torch.empty(256 << 20, dtype=torch.uint8, device=dev))
+        kw = dict(qo_indptr=c.indptr, paged_kv_indptr=c.kv_page_indptr, paged_kv_indices=c.kv_page_indices,
+                  paged_kv_last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D,
+                  page_size=P, qo_indptr_host=c.host["indptr"], paged_kv_indptr_host=c.host["kv_page_indptr"],
+                  paged_kv_last_page_len_host=c.host["kv_last_page_lens"],
+                  paged_kv_indices_host=c.host["kv_page_indices"])
+        w2.begin_forward(route_one_row_requests=False, **kw)
+        tiled_us = median_us(lambda l: w2.forward(wl.q[l], wl.pool.pages[l], causal=True))
+        w2.end_forward()
+        # the two halves alone: the decode rows as a batch of their own, the chunk as one
+        h = {k_: v_.numpy() for k_, v_ in c.host.items()}
+        i32 = lambda a_: torch.from_numpy(np.ascontiguousarray(a_, dtype=np.int32))
+        def sub_batch(lo, hi):
+            ip = h["kv_page_indptr"]
+            host = dict(qo_indptr_host=i32(h["indptr"][lo: hi + 1] - h["indptr"][lo]),
+                        paged_kv_indptr_host=i32(ip[lo: hi + 1] - ip[lo]),
+                        paged_kv_last_page_len_host=i32(h["kv_last_page_lens"][lo:hi]),
+                        paged_kv_indices_host=i32(h["kv_page_indices"][ip[lo]: ip[hi]]))
+            devs = {k_[:-5]: v_.to(dev) for k_, v_ in host.items()}
+            return dict(num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D, page_size=P, **devs, **host), \
+                slice(int(h["indptr"][lo]), int(h["indptr"][hi]))
+        halves = {}
+        for name, (lo, hi) in (("decode_rows", (0, n_dec)), ("chunk", (n_dec, len(wl.tasks)))):
+            kw_h, rows = sub_batch(lo, hi)
+            w2.begin_forward(**kw_h)
+            qh = wl.q[:, rows].contiguous()
+            halves[name] = median_us(lambda l: w2.forward(qh[l], wl.pool.pages[l], causal=True))
+            w2.end_forward()
+        dec_bytes = wl.decode_kv_tokens() * tok_bytes + 2 * n_dec * Hq * D * 2 + \
+            4 * int(h["kv_page_indptr"][n_dec])
+        flops = wl.chunk_flops()
+        out[tag] = {
+            "layers": L, "n_qo_heads": Hq, "decode_rows": n_dec, "rows_routed_to_decode_kernel": routed_rows,
+            "chunk_tokens": int(lens[0]), "chunk_prior": int(prior[0]), "chunk_parts_per_tile": parts,
+            "decode_kv_tokens": wl.decode_kv_tokens(), "kv_pages": n_pages,
+            "append_us_per_layer": round(append_us, 1),
+            "attention_us_per_layer": round(mixed_us, 1),
+            "attention_us_per_layer_all_rows_as_tiles": round(tiled_us, 1),
+            "decode_rows_alone_us_per_layer": round(halves["decode_rows"], 1),
+            "decode_rows_GBps": round(dec_bytes / halves["decode_rows"] / 1e3, 1),
+            "decode_rows_frac_of_hbm_peak": round(dec_bytes / halves["decode_rows"] / 1e3 / HBM_PEAK_GBPS, 4),
+            "chunk_alone_us_per_layer": round(halves["chunk"], 1),
+            "chunk_TFLOPs": round(flops / halves["chunk"] / 1e6, 1),
+            "chunk_frac_of_mfma_bf16_peak": round(flops / halves["chunk"] / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
+            "step_ms": round(step_ms, 3), "step_tokens_per_s": round(nnz / step_ms * 1e3, 1),
+            "whole_call_decode_bytes_GBps": round(dec_bytes / mixed_us / 1e3, 1),
+        }
+        del wl, w2, c
+        torch.cuda.empty_cache()
+    return out
 
 
 def fragmented_section(seed: int):
@@ -573,6 +776,24 @@ def fragmented_section(seed: int):
             "attention_frac_of_hbm_peak": round(attn_bytes / attn_us / 1e3 / HBM_PEAK_GBPS, 4)}
 
 
+def page8_in_child(seed: int):
+    """Configuration 2 on pages of 8 tokens - the page size the reference deploys with
+    (worker_api.py:170,187) - in a process of its own: the whole step and the attention pass."""
+    import subprocess
+
+    cmd = [sys.executable, os.path.abspath(__file__), "--page-size", "8", "--steps", "40", "--warmup", "6",
+           "--seed", str(seed), "--no-cpu-baseline", "--no-swap", "--no-prefill", "--no-fragmented",
+           "--no-graph", "--no-rope-step", "--no-mixed", "--no-page8"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"bench on 8-token pages failed with exit code {res.returncode}")
+    d = json.loads(res.stdout.strip().splitlines()[-1])
+    r = d.get("roofline", {})
+    return {"workload": d["config"]["workload"], "ms_per_step": d["ms_per_step"], "value_GBps": d["value"],
+            "pct_of_hbm_peak": d["pct_of_hbm_peak"], "attention_avg_launch_us": r.get("avg_launch_us"),
+            "attention_frac_of_hbm_peak": r.get("frac"), "steps": d["steps"]}
+
+
 def run_section_in_child(name: str, seed: int):
     """The host-link sections run in a process of their own, after this one has released the
     GPU memory it held: measured here, pinned-copy rates of a section depend on which streams
@@ -595,6 +816,10 @@ def main() -> int:
         if a.section == "prefill":
             print(json.dumps(prefill_section(a.seed, extras=not a.prefill_config4_only,
                                              config4=not a.prefill_one_chunk_only)))
+        elif a.section == "mfma-ceiling":
+            print(json.dumps(mfma_ceiling_section(a.seed)))
+        elif a.section == "mixed":
+            print(json.dumps(mixed_section(a.seed, shapes=tuple(a.mixed_shapes.split(",")))))
         else:
             print(json.dumps({"swap": swap_section, "fragmented": fragmented_section}[a.section](a.seed)))
         return 0
@@ -849,6 +1074,11 @@ def main() -> int:
     if not a.no_prefill:
         out["prefill"] = prefill_section(a.seed)
         torch.cuda.empty_cache()
+    if not a.no_mixed:
+        out["mixed"] = mixed_section(a.seed)
+        torch.cuda.empty_cache()
+    if not a.no_page8 and P == 16:
+        out["page8"] = page8_in_child(a.seed)
     if not a.no_swap:
         # three processes in a row: whether a swap overlaps with compute used to depend on the
         # process (which hardware queue its streams were given); the figures of all three are kept

@@ -22,7 +22,7 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     print("[case] bench.py line", flush=True)
     res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--steps", "4",
                           "--warmup", "1", "--no-swap", "--no-fragmented", "--no-prefill", "--no-graph",
-                          "--no-rope-step"], capture_output=True, text=True, timeout=300)
+                          "--no-rope-step", "--no-mixed", "--no-page8"], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stderr[-2000:]
     lines = [l for l in res.stdout.splitlines() if l.strip()]
     assert len(lines) == 1
@@ -37,7 +37,7 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     assert r["bound"] == "hbm" and r["peak"] == 8000.0 and r["unit"] == "GB/s"
     assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3 and 0.3 < r["frac"] < 1.0
     c = d["cpu_baseline"]
-    assert c["kind"] == "reference-restatement" and c["config"] == "configs[0]"
+    assert c["kind"] == "port" and c["config"] == "configs[0]"
     assert c["cores"] >= 1 and c["value"] > 0 and c["sample"]
     h = c["hip_same_config"]
     assert h["pages_bit_equal"] is True and h["max_rel_err_vs_cpu_per_request"] <= 1e-4 and h["us_per_step"] > 0
