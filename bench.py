@@ -74,8 +74,8 @@ def parse_args():
                     help="with --section prefill: only configuration 4's launches on its own data "
                          "(20 appends, 20 attention launches), for profiler runs whose per-kernel "
                          "averages must not mix in the zero-data and one-chunk measurements")
-    ap.add_argument("--mixed-shapes", default="8B,70B",
-                    help="with --section mixed: which stage shapes to run (8B, 70B)")
+    ap.add_argument("--mixed-shapes", default="8B,70B,8B_chunk_behind_8000",
+                    help="with --section mixed: which cases to run (8B, 70B, 8B_chunk_behind_8000)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="before the timed region run one plain page-copy kernel of known size "
                          "(256 MiB read + 256 MiB written) so counter runs can be scaled by it")
@@ -540,7 +540,7 @@ def mfma_ceiling_section(seed: int, levels=(0, 1, 2), fills=("normal", "constant
     return out
 
 
-def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
+def mixed_section(seed: int, shapes=("8B", "70B", "8B_chunk_behind_8000"), reps: int = 6):
     """The reference's usual step in its decode-first aggregated mode (engine/pipeline/stage/
     join.py:11-88, 512-token budget; deserve_exp/exp_args.csv: microbatch size 75): 75 running
     requests with contexts U[256, 4096], one new token each, plus one chunk that fills the
@@ -562,8 +562,10 @@ def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
     out = {"workload": "75 decode rows, ctx U[256,4096], + one 437-token chunk over a prior U[0,4096] (512-token "
                        "step budget), bf16, page 16, through the prefill wrapper; per layer"}
     for tag in shapes:
-        L, Hq = {"8B": (16, 32), "70B": (10, 64)}[tag]
+        L, Hq = {"8B": (16, 32), "70B": (10, 64), "8B_chunk_behind_8000": (16, 32)}[tag]
         dctx, prior, lens = mixed_step_shape(seed + 60)
+        if tag == "8B_chunk_behind_8000":
+            prior = [8000]          # a prompt as long as configuration 4's (the planner then shares the CUs)
         wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=seed + 61)
         n_dec, nnz = len(dctx), wl.nnz
         tok_bytes = wl.kv_bytes_per_token()
@@ -587,7 +589,9 @@ def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
             return ts[len(ts) // 2] * 1e3
 
         c = FlashPrefillCtx.init_and_plan(wl.tasks, wl.caches, w, Hq, Hkv, D, P)
-        routed_rows, parts = w._n_decode_rows, w._n_splits
+        routed_rows, parts, layout = w._n_decode_rows, w._n_splits, w._info.layout
+        launch_shape = {"decode_workgroups": w._info.n_decode_workgroups * (-(-Hkv // 4) if layout else 1),
+                        "tile_workgroups": w._n_tiles * Hkv, "waves_per_workgroup": 4 if layout else 8}
         n_pages = int(c.host["kv_page_indptr"][-1])
         append_us = median_us(lambda l: append_paged_kv_cache(wl.k[l], wl.v[l], c.indptr, wl.pool.pages[l],
                                                               c.kv_page_indices, c.kv_page_indptr,
@@ -621,6 +625,16 @@ def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
         w2.begin_forward(route_one_row_requests=False, **kw)
         tiled_us = median_us(lambda l: w2.forward(wl.q[l], wl.pool.pages[l], causal=True))
         w2.end_forward()
+        from deserve_amd import _lib
+        w2.begin_forward(route_one_row_requests=_lib.ROUTE_TWO_LAUNCHES, **kw)
+        two_us = median_us(lambda l: w2.forward(wl.q[l], wl.pool.pages[l], causal=True))
+        w2.end_forward()
+        w2.begin_forward(route_one_row_requests=_lib.ROUTE_SHARED_LAUNCH, **kw)
+        shared_us = median_us(lambda l: w2.forward(wl.q[l], wl.pool.pages[l], causal=True))
+        shared_shape = {"decode_workgroups": w2._info.n_decode_workgroups * -(-Hkv // 4),
+                        "tile_workgroups": w2._n_tiles * Hkv, "chunk_parts_per_tile": w2._n_splits,
+                        "waves_per_workgroup": 4}
+        w2.end_forward()
         # the two halves alone: the decode rows as a batch of their own, the chunk as one
         h = {k_: v_.numpy() for k_, v_ in c.host.items()}
         i32 = lambda a_: torch.from_numpy(np.ascontiguousarray(a_, dtype=np.int32))
@@ -645,11 +659,16 @@ def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
         flops = wl.chunk_flops()
         out[tag] = {
             "layers": L, "n_qo_heads": Hq, "decode_rows": n_dec, "rows_routed_to_decode_kernel": routed_rows,
+            "plan": "one launch, decode and tile workgroups share the compute units" if layout else
+                    ("all rows as query tiles" if routed_rows == 0 else "decode pass, then tile pass"),
+            "launch": launch_shape,
             "chunk_tokens": int(lens[0]), "chunk_prior": int(prior[0]), "chunk_parts_per_tile": parts,
             "decode_kv_tokens": wl.decode_kv_tokens(), "kv_pages": n_pages,
             "append_us_per_layer": round(append_us, 1),
             "attention_us_per_layer": round(mixed_us, 1),
             "attention_us_per_layer_all_rows_as_tiles": round(tiled_us, 1),
+            "attention_us_per_layer_decode_pass_then_tile_pass": round(two_us, 1),
+            "attention_us_per_layer_one_launch_shared_cus": round(shared_us, 1), "one_launch_shape": shared_shape,
             "decode_rows_alone_us_per_layer": round(halves["decode_rows"], 1),
             "decode_rows_GBps": round(dec_bytes / halves["decode_rows"] / 1e3, 1),
             "decode_rows_frac_of_hbm_peak": round(dec_bytes / halves["decode_rows"] / 1e3 / HBM_PEAK_GBPS, 4),
@@ -658,6 +677,8 @@ def mixed_section(seed: int, shapes=("8B", "70B"), reps: int = 6):
             "chunk_frac_of_mfma_bf16_peak": round(flops / halves["chunk"] / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
             "step_ms": round(step_ms, 3), "step_tokens_per_s": round(nnz / step_ms * 1e3, 1),
             "whole_call_decode_bytes_GBps": round(dec_bytes / mixed_us / 1e3, 1),
+            "whole_call_decode_bytes_frac_of_hbm_peak": round(dec_bytes / mixed_us / 1e3 / HBM_PEAK_GBPS, 4),
+            "whole_call_chunk_TFLOPs": round(flops / mixed_us / 1e6, 1),
         }
         del wl, w2, c
         torch.cuda.empty_cache()

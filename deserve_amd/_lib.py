@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libdskv.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 F32, F16, BF16 = 0, 1, 2
+ROUTE_OFF, ROUTE_AUTO, ROUTE_TWO_LAUNCHES, ROUTE_SHARED_LAUNCH = 0, 1, 2, 3
+LAYOUT_SEPARATE, LAYOUT_SHARED = 0, 1
 ABI_VERSION = 3          # DSKV_ABI_VERSION of the include/dskv.h these signatures were written against
 
 
@@ -23,7 +25,7 @@ class MixedPlanInfo(ctypes.Structure):
     """dskv_mixed_plan_t of include/dskv.h."""
     _fields_ = [("n_tiles", c_int32), ("n_splits", c_int32), ("n_tile_rows", c_int32),
                 ("n_decode_rows", c_int32), ("n_decode_items", c_int32), ("n_decode_workgroups", c_int32),
-                ("plan_words", c_int64), ("decode_plan_at", c_int64), ("row_map_at", c_int64),
+                ("layout", c_int32), ("reserved", c_int32), ("plan_words", c_int64), ("decode_plan_at", c_int64), ("row_map_at", c_int64),
                 ("tile_rows_at", c_int64), ("tile_workspace_bytes", c_int64),
                 ("decode_workspace_bytes", c_int64)]
 

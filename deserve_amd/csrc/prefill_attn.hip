@@ -29,571 +29,15 @@
 // a workgroup of its own that leaves (maximum, sum, unnormalised O) of its rows in a
 // workspace, and a merge pass (one workgroup per query row) turns the parts into the output.
 #include "kv_tile.h"
+#include "decode_kernel.h"
 
 #include <vector>
 
 #include <algorithm>
 
+#include "prefill_kernel.h"
+
 namespace dskv {
-
-#ifndef DSKV_PREFILL_WAVES
-#define DSKV_PREFILL_WAVES 8
-#endif
-#ifndef DSKV_PREFILL_COLTILES
-#define DSKV_PREFILL_COLTILES 1
-#endif
-constexpr int kPrefillWaves = DSKV_PREFILL_WAVES;   // waves per workgroup
-constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
-constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
-constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
-constexpr int kTileWords = 5;                       // plan entry: request, first row, block range, part
-constexpr int kRowsPerWave = kBlock / kPrefillWaves;   // rows of a block one wave loads
-constexpr int kRowGroups = kRowsPerWave / 4;           // in groups of 4 rows (one load each)
-static_assert(kRowsPerWave % 4 == 0 && kRowGroups >= 1, "a wave loads whole groups of 4 rows");
-// LDS layout of a 32-token block of K (or V) rows of one kv head: eight regions of four rows.
-// A region is what one load instruction delivers: 64 lanes x 16 bytes, lane p at byte 16 p.
-// Lane p = 4 c + rho fetches the 16-byte chunk c of row rho, so the region holds its rows
-// interleaved chunk by chunk ((4 c + rho) * 16); regions are 1088 bytes apart (64 bytes of
-// padding).  Operand reads are free of bank conflicts: the 16 lanes of a K-operand read (16
-// token rows, one chunk) and the 32 lanes of a transposing V read (4 rows x 4 chunks of a
-// region) fall on 16 different 16-byte bank groups each.
-constexpr int kRegionBytes = 1088;
-constexpr int kStageBytes = (kBlock / 4) * kRegionBytes;
-// The running maximum of a column is only raised when a block exceeds it by more
-// than this (log2 domain): probabilities stay below 2^8, the accumulators are
-// rescaled a handful of times per query instead of once per block.
-constexpr float kRescaleSlack = 8.f;
-#ifndef DSKV_PREFILL_KREADS_FIRST
-#define DSKV_PREFILL_KREADS_FIRST 0
-#endif
-#ifndef DSKV_PREFILL_SUM_ON_MFMA
-#define DSKV_PREFILL_SUM_ON_MFMA 0
-#endif
-constexpr bool kSumOnMfma = DSKV_PREFILL_SUM_ON_MFMA;   // row sums of P by the matrix pipeline
-
-// Lane roles of the 32x32x16 MFMA, with h = lane / 32 and r = lane % 32:
-//   A operand: row r, k = 8h .. 8h+7.   B operand: column r, k = 8h .. 8h+7.
-//   C/D: column r, rows 8i + 4h + j in register 4i + j (i, j = 0..3).
-template <int DT, bool kRowsSharePage>
-#ifndef DSKV_PREFILL_MIN_WAVES
-#define DSKV_PREFILL_MIN_WAVES 1
-#endif
-__global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void prefill_attn_mfma_kernel(
-    uint16_t *__restrict__ out, const uint16_t *__restrict__ q,
-    const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
-    const int32_t *__restrict__ kv_indices, const int32_t *__restrict__ kv_indptr,
-    const int32_t *__restrict__ kv_last, const int32_t *__restrict__ tile_info, int n_qo_heads,
-    int n_kv_heads, int page_shift, float scale_log2, int causal, int n_splits,
-    float *__restrict__ part_o, float *__restrict__ part_ml, int max_slots)
-{
-    typedef Elt<DT> E;
-    __shared__ __align__(16) char k_stage[4][kStageBytes];
-    __shared__ __align__(16) char v_stage[4][kStageBytes];
-
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    const int g = lane >> 4;     // row group / chunk roles of the K/V row movement
-    const int c = lane & 15;
-    const int h = lane >> 5;     // MFMA roles
-    const int r = lane & 31;
-    const int kvh = blockIdx.x % n_kv_heads;
-    const int tile = blockIdx.x / n_kv_heads;
-    const int group = n_qo_heads / n_kv_heads;
-    const int pos_per_wave = kWaveCols / group;    // query positions per wave
-
-    // plan entry: request, first query row of the tile within it, and the 32-token blocks
-    // [blk_begin, blk_end) of the request's K/V that this workgroup walks (all of them unless
-    // the plan splits tiles; blk_begin is a multiple of four), as part `split` of n_splits
-    const const_i32_ptr entry = as_const(tile_info) + (long)tile * kTileWords;
-    const int b = entry[0];
-    const int q0 = entry[1];
-    const int blk_begin = entry[2];
-    const int kv_cap_blocks = entry[3];
-    const int split = entry[4];
-    const int q_begin = qo_indptr[b];
-    const int n_b = qo_indptr[b + 1] - q_begin;
-    const int n_pages = kv_indptr[b + 1] - kv_indptr[b];
-    const int kv_len = n_pages > 0 ? ((n_pages - 1) << page_shift) + kv_last[b] : 0;
-    // tokens this workgroup may look at end here: the request's end, or the end of its part
-    const int kv_cap = min(kv_len, kv_cap_blocks < (1 << 25) ? kv_cap_blocks * kBlock : kv_len);
-    const_i32_ptr page_ids = as_const(kv_indices) + kv_indptr[b];
-    const int row_bytes = n_kv_heads * kHeadDim * 2;
-    const int half_bytes = row_bytes << page_shift;
-    const long page_bytes = 2L * half_bytes;
-    const int page_mask = (1 << page_shift) - 1;
-
-    // column r of column tile ct: query row wq0 + (32 ct + r)/group, head (32 ct + r)%group
-    const int wq0 = q0 + wave * pos_per_wave;
-    int qrow[kColTiles], c_head[kColTiles], limit[kColTiles];   // limit: kv tokens the column may see
-    bool live[kColTiles];
-    u32x4 qreg[kColTiles][8];     // dims 16*ks + 8h .. +7 of the column's query
-#pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        const int col = 32 * ct + r;
-        const int c_pos = col / group;
-        c_head[ct] = col - c_pos * group;
-        qrow[ct] = wq0 + c_pos;
-        live[ct] = c_pos < pos_per_wave && qrow[ct] < n_b;
-        const int lim = causal ? kv_len - n_b + qrow[ct] + 1 : kv_len;
-        limit[ct] = live[ct] ? min(max(lim, 0), kv_cap) : 0;
-        const uint16_t *qrow_p =
-            q + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim + h * 8;
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            u32x4 z = {0, 0, 0, 0};
-            qreg[ct][ks] = live[ct] ? *reinterpret_cast<const u32x4 *>(qrow_p + ks * 16) : z;
-        }
-    }
-    // Token ranges from scalars only: they steer loops, barriers and page lookups
-    // and must be uniform for the compiler too.  The workgroup walks [0, t_end);
-    // a wave computes on [0, w_end) and masks from w_mask_from on.
-    const int rows_wg = min(kPrefillWaves * pos_per_wave, n_b - q0);          // >= 1 by construction
-    const int t_first = blk_begin * kBlock;                                   // the walk starts here
-    const int t_end = min(max(causal ? kv_len - n_b + q0 + rows_wg : kv_len, 0), kv_cap);
-    const int rows_w = min(pos_per_wave, n_b - wq0);                          // <= 0: idle wave
-    const int w_mask_from =
-        rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + 1 : kv_len, 0), kv_cap) : 0;
-    int w_end = rows_w > 0 ? min(max(causal ? kv_len - n_b + wq0 + rows_w : kv_len, 0), kv_cap) : 0;
-    if (w_end <= t_first) w_end = 0;   // nothing of this part is visible to the wave's rows: idle
-
-    const int n_blocks = (t_end + kBlock - 1) / kBlock;
-    // Start value of the running maximum: far below any scaled score, far above a
-    // scaled masked score (kNegBig * scale_log2).
-    float m_run[kColTiles];
-    f32x16 acc[kColTiles][4];     // O^T: dims 32*dt + 8i + 4h + j of column r in acc[ct][dt][4i + j]
-    // Row sums of P, optionally on the matrix pipeline: ones(32 x tokens) . P^T - every
-    // register of a lane then holds the sum of its column r over the tokens multiplied so
-    // far.  It takes 16 additions per block off the vector pipeline and adds two MFMAs;
-    // measured on MI355X the kernel takes the same time either way, so the default keeps the
-    // sums on the vector pipeline (fewer registers, less matrix work).
-    f32x16 l_acc[kColTiles];
-    float l_run[kColTiles];       // the same sums kept by the vector pipeline (kSumOnMfma off)
-    u32x4 pb[kColTiles][2];       // packed probabilities of the previous block, per k-step
-#pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        m_run[ct] = 0.5f * kNegBig * scale_log2;
-        l_run[ct] = 0.f;
-#pragma unroll
-        for (int v = 0; v < 16; v++) l_acc[ct][v] = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[ct][dt][v] = 0.f;
-        pb[ct][0] = pb[ct][1] = u32x4{0, 0, 0, 0};
-    }
-    const uint32_t one2 = E::pack2(1.f, 1.f);
-    const u32x4 ones = {one2, one2, one2, one2};
-
-    // A plan that splits tiles: every part leaves (max, sum, unnormalised O) of its rows in
-    // slot row * n_splits + split of the workspace (O blocks of all slots, then their (max,
-    // sum) pairs); a part that sees nothing leaves zeros and a maximum below any real one.
-    auto store_partial = [&](int ct, float m, float l) {
-        const long slot = (long)(q_begin + qrow[ct]) * n_splits + split;
-        if (slot >= max_slots) return;   // a slot beyond the workspace is never written
-        const long qh = (long)kvh * group + c_head[ct];
-        float *o = part_o + (slot * n_qo_heads + qh) * kHeadDim + 4 * h;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                *reinterpret_cast<f32x4 *>(o + dt * 32 + 8 * i) =
-                    f32x4{acc[ct][dt][4 * i], acc[ct][dt][4 * i + 1], acc[ct][dt][4 * i + 2], acc[ct][dt][4 * i + 3]};
-        if (h == 0) {
-            float *ml = part_ml + (slot * n_qo_heads + qh) * 2;
-            ml[0] = m;
-            ml[1] = l;
-        }
-    };
-    // No kv token of this part visible to any row of the tile: the output rows are zero
-    // (or the part is empty).  Uniform over the workgroup, and before the first barrier.
-    if (t_end <= t_first) {
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            if (!live[ct]) continue;
-            if (n_splits > 1) {
-                store_partial(ct, m_run[ct], 0.f);
-                continue;
-            }
-            uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
-                          4 * h;
-#pragma unroll
-            for (int i = 0; i < 16; i++) *reinterpret_cast<u32x2 *>(o + 8 * i) = u32x2{0, 0};
-        }
-        return;
-    }
-
-    // This wave's share of the K (or V) rows of block blk: rows wave*kRowsPerWave .. +kRowsPerWave,
-    // in groups of four (one region each).  Rows at or past t_end arrive as zeros (their
-    // probabilities are zero, but 0 * garbage is not).
-    //
-    // Pages of at least four tokens (kRowsSharePage): the rows go from memory straight into
-    // their LDS region (buffer_load ... lds: lane p's 16 bytes land at region + 16 p, lanes
-    // beyond the descriptor's end write zeros), addressed through descriptors that end after
-    // the group's last valid row.  Page ids are looked up with a vector load (every lane the
-    // same entry; entries past the table read as page 0, whose descriptor is then empty).
-    // Smaller pages: every lane resolves its own page, the rows pass through registers.
-    typedef __attribute__((address_space(3))) void *lds_ptr;
-    const int direct_off = (lane & 3) * row_bytes + kvh * (kHeadDim * 2) + (lane >> 2) * 16;
-    const int lane_off = kvh * (kHeadDim * 2) + c * 16;
-    // Page ids come through scalar loads (block-table entries past the table are clamped to
-    // its last one; their descriptors are empty).  They are consumed at the end of an
-    // iteration, when every LDS read of the iteration has been waited for anyway (scalar
-    // loads and LDS reads share a counter).
-    const int last_entry = max(n_pages - 1, 0);
-    auto lookup_pages = [&](int blk, int(&pg)[kRowGroups]) {
-        if (!kRowsSharePage) return;
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++) {
-            const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
-            pg[i] = page_ids[min(tok0 >> page_shift, last_entry)];
-        }
-    };
-    // The descriptors of the rows of block blk (scalar work: page id into an SGPR, base
-    // address, valid bytes), prepared an iteration before the loads are issued so that it
-    // runs in the shadow of that iteration's MFMAs.
-    struct RowDesc {
-        u32x4 k[kRowGroups], v[kRowGroups];   // raw buffer descriptors: base, base >> 32, bytes, flags
-    };
-    auto make_desc = [&](const char *base, int bytes) {
-        const uint64_t a = (uint64_t)base;
-        return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
-                     (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xFFFFu)),
-                     (uint32_t)__builtin_amdgcn_readfirstlane(bytes), (uint32_t)kBufferFlags};
-    };
-    auto prepare_rows = [&](int blk, const int(&pg)[kRowGroups], RowDesc &d) {
-        if (!kRowsSharePage) return;
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++) {
-            const int tok0 = blk * kBlock + wave * kRowsPerWave + 4 * i;
-            // one page holds the 4 rows: descriptors that end after the last
-            // valid row make the bounds check free and keep offsets constant
-            // (the clamp is selected as a vector instruction: back to a scalar register, the
-            // descriptor words must live in SGPRs)
-            const int valid = __builtin_amdgcn_readfirstlane(min(max(t_end - tok0, 0), 4));
-            const char *first_row = pages + (long)pg[i] * page_bytes + (long)(tok0 & page_mask) * row_bytes;
-            d.k[i] = make_desc(first_row, valid * row_bytes);
-            d.v[i] = make_desc(first_row + half_bytes, valid * row_bytes);
-        }
-    };
-    auto region_of = [&](char *stage, int i) { return stage + (wave * kRowGroups + i) * kRegionBytes; };
-    // Written out as instructions: through the compiler's builtin every later LDS read waits
-    // for ALL of these loads (it cannot tell which region a read touches), which would undo
-    // requesting them three iterations early.  What it does not know it does not wait for:
-    // the waits for these loads are the explicit ones below.
-    // M0 is on the clobber list (the compiler reserves it, sets it itself before the few
-    // instructions that read it, and must not assume that such a setting survives this one).
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-    auto load_direct = [&](const u32x4(&rows)[kRowGroups], char *stage) {
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++) {
-            const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_ptr)region_of(stage, i);
-            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                         :
-                         : "s"(lds_addr), "v"(direct_off), "s"(rows[i])
-                         : "memory", "m0");
-        }
-    };
-#pragma clang diagnostic pop
-    auto load_rows = [&](int blk, u32x4(&k_rows)[kRowGroups], u32x4(&v_rows)[kRowGroups]) {
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++) {
-            const int tok = blk * kBlock + wave * kRowsPerWave + 4 * i + g;
-            const int tc = max(min(tok, t_end - 1), 0);
-            const char *p = pages + page_ids[tc >> page_shift] * page_bytes +
-                            (long)(tc & page_mask) * row_bytes + lane_off;
-            const u32x4 z = {0, 0, 0, 0};
-            const u32x4 got_k = *reinterpret_cast<const u32x4 *>(p);
-            const u32x4 got_v = *reinterpret_cast<const u32x4 *>(p + half_bytes);
-            k_rows[i] = tok < t_end ? got_k : z;
-            v_rows[i] = tok < t_end ? got_v : z;
-        }
-    };
-    auto store_rows = [&](char *stage, const u32x4(&rows)[kRowGroups]) {   // lane (g, c): chunk c of row g
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++)
-            *reinterpret_cast<u32x4 *>(region_of(stage, i) + (c * 4 + g) * 16) = rows[i];
-    };
-    // Waits until at most n of this wave's vector-memory operations are outstanding (the
-    // other counters of s_waitcnt left at "do not wait").
-#define DSKV_WAIT_VMEM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | 0x70 | 0xF00 | (((n) >> 4) << 14))
-
-    // Two score buffers that the iterations use in turn (S(m) is still being turned into
-    // P(m) while S(m+1) is computed): the loop is unrolled with static phases, so which
-    // buffer is which is known at compile time and no copy is needed.
-    f32x16 xs[2][kColTiles];
-    u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
-    auto read_k_operands = [&](const char *kst) {
-        // token r = row r & 3 of region r >> 2; chunk 2 ks + h
-        const char *k_rows = kst + (r >> 2) * kRegionBytes + h * 64 + (r & 3) * 16;
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 128);
-    };
-    auto scores = [&](int buf) {
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) xs[buf][ct][v] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++)
-#pragma unroll
-            for (int ct = 0; ct < kColTiles; ct++)
-                xs[buf][ct] = E::mfma_32x32(ka[ks], qreg[ct][ks], xs[buf][ct]);
-    };
-    // Masks block blk's scores (needed from w_mask_from on).  The empty volatile statement
-    // keeps this a branch: the compiler otherwise turns it into selects that every block
-    // pays for (48 vector instructions), and only the blocks on the diagonal need it.
-    auto mask_scores = [&](int blk, int buf) {
-        const int t = blk * kBlock;
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            asm volatile("" : "+v"(xs[buf][ct]));   // (re)defined here: the selects cannot leave the branch
-#pragma unroll
-            for (int v = 0; v < 16; v++)
-                if (t + 8 * (v >> 2) + 4 * h + (v & 3) >= limit[ct]) xs[buf][ct][v] = kNegBig;
-        }
-    };
-    // Column maximum of the block in xs[buf], and whether the running maximum has to be
-    // raised before the block's exponentials.
-    float m_blk[kColTiles];
-    bool raise = false;
-    auto block_max = [&](int buf) {
-        raise = false;
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            const f32x16 &xc = xs[buf][ct];
-            // scale_log2 > 0: the maximum can be taken before scaling.  A chain of
-            // three-input maxima: 8 instructions for 16 values.
-            float m = fmaxf(fmaxf(xc[0], xc[1]), xc[2]);
-#pragma unroll
-            for (int v = 3; v < 15; v += 2) m = fmaxf(fmaxf(m, xc[v]), xc[v + 1]);
-            m = fmaxf(m, xc[15]);
-            float other = m;
-            swap_halves32(m, other);
-            m_blk[ct] = fmaxf(m, other) * scale_log2;
-            raise |= m_blk[ct] > m_run[ct] + kRescaleSlack;
-        }
-    };
-
-    // Iteration m of the main loop multiplies P(m-1) into V(m-1), turns S(m) into
-    // P(m) and computes S(m+1), so that every MFMA of the iteration is independent
-    // of its exponentials and the matrix and vector pipelines of a wave overlap.
-    // Block j lives in K stage j % 4 and V stage j % 4.  Per iteration one barrier; every
-    // wave runs every iteration (idle ones only move rows), so the barriers match.  The loop
-    // is unrolled by four so that all stage indices are static.
-    //   Direct path: iteration m requests K(m+3) and V(m+2) behind its barrier (K(m+3)
-    //   replaces K(m-1), last read in iteration m-2; V(m+2) replaces V(m-2), last read in
-    //   iteration m-1).  K(m+1), which iteration m reads, went out two iterations earlier; a
-    //   wave makes sure that its own part of it has landed (at most 3 younger loads per row
-    //   group outstanding: V(m), K(m+2), V(m+1)) before it joins the barrier
-    //   that publishes the block.  The page of block j is looked up in iteration j-5 and its
-    //   descriptors are built in iteration j-4, behind that iteration's MFMAs.
-    //   Register path: the rows of block m+4 are requested in iteration m and written to
-    //   LDS in iteration m+2 (one iteration is shorter than a trip to memory).
-    RowDesc desc[4];              // descriptors of block j in desc[j % 4]
-    int pg[4][kRowGroups];        // page ids of block j in pg[j % 4]
-    struct RowSet {
-        u32x4 k[kRowGroups], v[kRowGroups];   // rows on their way to LDS (register path)
-    };
-    RowSet even, odd;
-    {
-        const u32x4 z = {0, 0, 0, 0};
-        u32x4 zero[kRowGroups];
-#pragma unroll
-        for (int i = 0; i < kRowGroups; i++) zero[i] = z;
-        store_rows(v_stage[3], zero);   // V(-1): multiplied by P(-1) = 0, must be finite
-        // the walk starts at block blk_begin, a multiple of four: block j still lives in stage j % 4
-        if (kRowsSharePage) {
-#pragma unroll
-            for (int blk = 0; blk < 4; blk++) lookup_pages(blk_begin + blk, pg[blk]);
-#pragma unroll
-            for (int blk = 0; blk < 4; blk++) prepare_rows(blk_begin + blk, pg[blk], desc[blk]);
-#pragma unroll
-            for (int blk = 0; blk < 3; blk++) load_direct(desc[blk].k, k_stage[blk]);
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) load_direct(desc[blk].v, v_stage[blk]);
-            lookup_pages(blk_begin + 4, pg[0]);
-            DSKV_WAIT_VMEM(0);
-        } else {
-            u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) load_rows(blk_begin + blk, first_k[blk], first_v[blk]);
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                store_rows(k_stage[blk], first_k[blk]);
-                store_rows(v_stage[blk], first_v[blk]);
-            }
-            load_rows(blk_begin + 2, even.k, even.v);
-            load_rows(blk_begin + 3, odd.k, odd.v);
-        }
-    }
-    __syncthreads();
-    if (w_end > 0) {
-        read_k_operands(k_stage[0]);
-        scores(0);
-        if ((blk_begin + 1) * kBlock > w_mask_from) mask_scores(blk_begin, 0);
-        block_max(0);
-    }
-    // V operand: token 16 ks + 8 hi + 4 h + (c >> 2) = row c >> 2 of region 4 ks + 2 hi + h;
-    // bytes 64 dt + 32 (g & 1) + 8 (c & 3) of its row = half (c & 1) of chunk 4 dt + 2 (g & 1) + ((c & 3) >> 1)
-    const int v_lane_off = h * kRegionBytes + (2 * (g & 1) + ((c & 3) >> 1)) * 64 + (c >> 2) * 16 + (c & 1) * 8;
-    auto iteration = [&](int m, int phase, RowSet &rows) {   // phase = m % 4, a literal at each call
-        if (kRowsSharePage) {
-            // this wave's rows of K(m+1) have landed; then the bare barrier: with the fences of
-            // __syncthreads the compiler waits for EVERY load into LDS still on its way, which
-            // is the whole point of requesting them early.  Nothing else needs the fences here:
-            // the loop of this path writes LDS through these loads only, and the LDS reads of
-            // the previous iteration have been consumed.
-            // (the empty statements pin the compiler's order of ordinary LDS accesses around the
-            // barrier, which the builtin by itself does not: the previous iteration's operand
-            // reads stay above it, this iteration's below)
-            DSKV_WAIT_VMEM(3 * kRowGroups);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-        } else {
-            __syncthreads();
-        }
-        if (kRowsSharePage) {
-            lookup_pages(m + 5, pg[(phase + 1) & 3]);
-            load_direct(desc[(phase + 3) & 3].k, k_stage[(phase + 3) & 3]);   // K(m+3)
-            load_direct(desc[(phase + 2) & 3].v, v_stage[(phase + 2) & 3]);   // V(m+2)
-        } else {
-            store_rows(k_stage[(phase + 2) & 3], rows.k);                     // K(m+2)
-            store_rows(v_stage[(phase + 2) & 3], rows.v);                     // V(m+2)
-            load_rows(m + 4, rows.k, rows.v);
-        }
-        if (!(w_end > 0 && (m - 1) * kBlock < w_end)) {
-            prepare_rows(m + 4, pg[phase], desc[phase]);
-            return;
-        }
-        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-            // rare: raise the maximum and bring what was computed under the old
-            // one (accumulators, row sum, the pending P(m-1)) to the new scale
-#pragma unroll
-            for (int ct = 0; ct < kColTiles; ct++) {
-                const float m_new = fmaxf(m_run[ct], m_blk[ct]);
-                const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
-                m_run[ct] = m_new;
-                if (kSumOnMfma) l_acc[ct] *= alpha;
-                else l_run[ct] *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < 4; dt++) acc[ct][dt] *= alpha;
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                    for (int w = 0; w < 4; w++) {
-                        float lo, hi;
-                        E::unpack2(pb[ct][ks][w], lo, hi);
-                        pb[ct][ks][w] = E::pack2(lo * alpha, hi * alpha);
-                    }
-            }
-        }
-        // The rest of the iteration is two straight-line halves, each an MFMA
-        // strand with independent vector work in its shadow:
-        //   S(m+1) = K(m+1).Q^T     |  P(m) = exp2(S(m) * scale - max), packed; row sum;
-        //                           |  V(m-1) operands from LDS
-        //   O += P(m-1).V(m-1)      |  maximum of S(m+1)
-        // with the masking of S(m+1), where needed, between them.  A masked score
-        // is kNegBig and the maximum never drops below its start value, so masked
-        // probabilities come out as exp2(-huge) = 0 without a select.
-        const int cur = phase & 1, nxt = cur ^ 1;   // xs[cur] = S(m), xs[nxt] receives S(m+1)
-        u32x4 pb_prev[kColTiles][2];
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            pb_prev[ct][0] = pb[ct][0];
-            pb_prev[ct][1] = pb[ct][1];
-        }
-        // V operand: the transposing read hands each block of 16 lanes four tokens
-        // of 16 consecutive dims, lane i of the block supplying the address of dims
-        // 4*(i%4) .. +3 of the block's token i/4
-        read_k_operands(k_stage[(phase + 1) & 3]);                       // K(m+1)
-#if DSKV_PREFILL_KREADS_FIRST
-        __builtin_amdgcn_sched_barrier(0);   // all eight K operands requested before anything else
-#endif
-        const char *v_rows = v_stage[(phase + 3) & 3] + v_lane_off;        // V(m-1)
-        u32x4 va[4][2];
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                const char *vp = v_rows + ks * 4 * kRegionBytes + dt * 256;
-                const u32x2 a_lo = read_transposed(vp);
-                const u32x2 a_hi = read_transposed(vp + 2 * kRegionBytes);
-                va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
-            }
-        scores(nxt);
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) {
-            float p[16], p_sum = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(xs[cur][ct][v], scale_log2, -m_run[ct]));
-                if (!kSumOnMfma) p_sum += p[v];
-            }
-            if (!kSumOnMfma) l_run[ct] += p_sum;
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-                pb[ct][ks] = u32x4{E::pack2(p[8 * ks], p[8 * ks + 1]), E::pack2(p[8 * ks + 2], p[8 * ks + 3]),
-                                   E::pack2(p[8 * ks + 4], p[8 * ks + 5]), E::pack2(p[8 * ks + 6], p[8 * ks + 7])};
-            // keeps P(m) in this half (it is only consumed by the next iteration)
-            asm volatile("" ::"v"(pb[ct][0]), "v"(pb[ct][1]), "v"(l_run[ct]));
-        }
-        if ((m + 2) * kBlock > w_mask_from) mask_scores(m + 1, nxt);   // wave-uniform
-
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                for (int ct = 0; ct < kColTiles; ct++)
-                    acc[ct][dt] = E::mfma_32x32(va[dt][ks], pb_prev[ct][ks], acc[ct][dt]);
-        if (kSumOnMfma)
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                for (int ct = 0; ct < kColTiles; ct++)
-                    l_acc[ct] = E::mfma_32x32(ones, pb_prev[ct][ks], l_acc[ct]);
-        prepare_rows(m + 4, pg[phase], desc[phase]);   // for the loads of the next iterations
-        block_max(nxt);
-#pragma unroll
-        for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
-    };
-    for (int m = blk_begin; m <= n_blocks; m += 4) {
-        iteration(m, 0, even);
-        iteration(m + 1, 1, odd);
-        iteration(m + 2, 2, even);
-        iteration(m + 3, 3, odd);
-    }
-    if (kRowsSharePage) DSKV_WAIT_VMEM(0);   // nothing of this wave may still be on its way into LDS
-#undef DSKV_WAIT_VMEM
-
-#pragma unroll
-    for (int ct = 0; ct < kColTiles; ct++) {
-        float l = l_acc[ct][0];   // summed over all tokens by the MFMA (both lane halves)
-        if (!kSumOnMfma) {
-            float l_other = l_run[ct];
-            swap_halves32(l_run[ct], l_other);
-            l = l_run[ct] + l_other;
-        }
-        if (!live[ct]) continue;
-        if (n_splits > 1) {
-            store_partial(ct, m_run[ct], l);
-            continue;
-        }
-        const float inv = l > 0.f ? 1.f / l : 0.f;
-        uint16_t *o = out + ((long)(q_begin + qrow[ct]) * n_qo_heads + (long)kvh * group + c_head[ct]) * kHeadDim +
-                      4 * h;
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                u32x2 w = {E::pack2(acc[ct][dt][4 * i] * inv, acc[ct][dt][4 * i + 1] * inv),
-                           E::pack2(acc[ct][dt][4 * i + 2] * inv, acc[ct][dt][4 * i + 3] * inv)};
-                *reinterpret_cast<u32x2 *>(o + dt * 32 + 8 * i) = w;
-            }
-    }
-}
 
 // Generic path (fp32 pools, head_dim != 128, group > 16): one wavefront per
 // (query row, q head), plain VALU, sequential over the visible tokens.
@@ -743,10 +187,75 @@ __global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
     }
 }
 
-static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads)
+static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads, int waves)
 {
     const int group = n_qo_heads / n_kv_heads;
-    return group <= kWaveCols ? kPrefillWaves * (kWaveCols / group) : 1;
+    return group <= kWaveCols ? waves * (kWaveCols / group) : 1;
+}
+
+// ---------------------------------------------------------------------------
+// The mixed launch: decode workgroups and query tiles side by side on every CU.
+//
+// A compute unit moves at most ~36 GB/s through its vector memory path (measured: one
+// decode workgroup of eight, four or two waves per CU streams 37, 35 and 31 GB/s, whatever
+// else is free), so the chip's 8 TB/s are only there when EVERY CU has loads in flight -
+// and a CU that computes a chunk's query tiles (bound by its matrix pipeline) contributes
+// none.  Run one after the other, the decode rows and the chunk of a mixed step (75 rows over
+// U[256,4096] tokens + 437 tokens over 2506) take 118 + 47 us; as tiles of one launch, with
+// one live row per 64-row tile and the longest rows walked by a single workgroup, 147 us
+// (228 us when the chunk follows 8000 tokens).  Here both kinds of work are workgroups of
+// FOUR waves (one per SIMD, at most 256 vector registers, half a CU's LDS each), so two fit
+// on a CU, and the launch starts with one decode workgroup per CU: the dispatcher places the
+// first #CU workgroups of a grid one per CU (measured on the box), so the decode workgroups -
+// statically balanced shares that must all start at once - own one slot of every CU for the
+// whole launch, while the query tiles pass through the other slot.  Measured: 150 us (175 us
+// behind 8000 tokens): the tile workgroups finish within 66 us, the decode workgroups, which
+// share the CU's memory path with them meanwhile, after 145 us instead of 113 us alone.
+// ---------------------------------------------------------------------------
+// Tiles in flight per decode wave of the mixed launch (2, 4 and 5 measured the same).
+constexpr int kSharedRing = kStages;
+// Wave priority of the tile workgroups.  At equal priority the compute unit serves the older
+// waves first, and the decode waves - launched first, never short of a load to issue - kept
+// the tile waves' few loads waiting: a tile workgroup took 162 us beside them instead of 38 us
+// alone.  With the tile waves ahead (any priority above 0) it takes 66 us.
+constexpr int kSharedTilePriority = 3;
+struct MixedArgs {
+    uint16_t *out;
+    const uint16_t *q;
+    const char *pages;
+    const int32_t *kv_indices;
+    int n_qo_heads, n_kv_heads, page_shift;
+    float scale_log2;
+    // decode side: shares x head groups workgroups come first in the grid
+    const Item *items;
+    const int32_t *wg_ptr;
+    float *dec_part_o, *dec_part_ml;
+    int dec_max_slots, n_decode_wgs, head_groups;
+    // tile side
+    const int32_t *qo_indptr, *kv_indptr, *kv_last, *tile_info;
+    float *tile_part_o, *tile_part_ml;
+    int tile_max_slots, n_splits, causal;
+};
+
+template <int DT, int kPagesPerTile>
+__global__ __launch_bounds__(64 * kSharedWaves, 2) void mixed_attn_kernel(const MixedArgs a)
+{
+    static_assert(kSharedWaves == kPrefillWavesShared, "both kinds of workgroup have the launch's size");
+    static_assert(kPrefillLdsBytes >= kSharedWaves * kVTileBytes, "the LDS is shared by the two bodies");
+    __shared__ __align__(16) char lds[kPrefillLdsBytes];
+    const int wg = blockIdx.x;
+    if (wg < a.n_decode_wgs)
+        decode_attn_body<DT, kPagesPerTile, kSharedWaves, kSharedRing>(
+            lds, wg / a.head_groups, wg % a.head_groups, a.out, a.q, a.pages, a.kv_indices, a.items, a.wg_ptr,
+            a.dec_part_o, a.dec_part_ml, a.dec_max_slots, a.n_qo_heads, a.n_kv_heads, a.page_shift,
+            a.scale_log2, nullptr, nullptr, nullptr);
+    else {
+        __builtin_amdgcn_s_setprio(kSharedTilePriority);
+        prefill_attn_body<DT, true, kPrefillWavesShared>(
+            lds, wg - a.n_decode_wgs, a.out, a.q, a.qo_indptr, a.pages, a.kv_indices, a.kv_indptr, a.kv_last,
+            a.tile_info, a.n_qo_heads, a.n_kv_heads, a.page_shift, a.scale_log2, a.causal, a.n_splits,
+            a.tile_part_o, a.tile_part_ml, a.tile_max_slots);
+    }
 }
 
 }  // namespace dskv
@@ -760,6 +269,11 @@ constexpr int kMaxPrefillSplits = 8;         // parts a tile's K/V range is cut 
 constexpr int kMinSplitTokens = 512;
 constexpr int kMaxSplitTarget = 1024;        // workgroups a split plan aims at, at most
 constexpr int32_t kWholeRange = 0x7fffffff;  // blk_end of a tile that is not split
+// kv tokens the one-row requests of a mixed batch must hold together before they get decode
+// workgroups of their own beside the tiles (64 MB of K/V per layer in the 8-kv-head bf16 shape)
+constexpr int64_t kMinSharedLaunchTokens = 16384;
+// ... and kv tokens the longest tiled request must hold (see dskv_mixed_plan)
+constexpr int64_t kMinSharedLaunchTiledKeys = 4096;
 
 static int compute_units()
 {
@@ -790,9 +304,9 @@ static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
                       int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
                       int32_t target_workgroups, int32_t *plan_host, int64_t capacity_words,
                       int32_t *n_tiles_out, int32_t *n_splits_out, int64_t *plan_words_out,
-                      int64_t *workspace_bytes_out)
+                      int64_t *workspace_bytes_out, int waves = kPrefillWaves)
 {
-    const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads);
+    const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads, waves);
     // later query tiles of a request see more keys: they come first within a request
     struct Tile { int32_t b, row; int64_t keys; };
     std::vector<Tile> tiles;
@@ -921,6 +435,8 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     // One query row under the end-aligned mask sees every kv token of its request, with or
     // without the mask: exactly a decode row.  Routed only where the 16-bit decode kernel
     // takes the shape; a request without kv tokens stays with the tiles (a row of zeros).
+    DSKV_REQUIRE(route_one_row_requests >= 0 && route_one_row_requests <= DSKV_ROUTE_SHARED_LAUNCH,
+                 "mixed_plan: unknown routing mode %d", route_one_row_requests);
     const bool route = route_one_row_requests && decode_mfma_shape(head_dim, n_qo_heads, n_kv_heads, page_size);
     std::vector<int32_t> kv_len(batch);
     std::vector<char> routed(batch, 0);
@@ -944,10 +460,40 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
             for (int64_t i = 0; i < n_b; i++) tile_rows.push_back((int32_t)(qo_indptr_host[b] + i));
         }
     }
+    // How the routed rows run.  Without tiled rows: the decode kernel by itself (workgroups of
+    // eight waves; 117 us where the same rows take 138 us as tiles).  With both kinds: one
+    // launch of four-wave workgroups that share the CUs (pages of at least four tokens: the
+    // tile side then loads straight into LDS) - if the decode rows are worth it (a handful of
+    // short decode rows beside a large batch of chunks stay tiles of the usual launch) and if
+    // a chunk follows a long context: as tiles of one launch, a chunk's 64 rows walk all
+    // their keys in ONE workgroup, and behind 8000 tokens that walk outlasts everything else
+    // (228 us against 175 us shared); behind 2500 tokens the two forms take the same time
+    // (144 and 141 + 10 us of merges), and the plain tiles are kept.
+    int64_t routed_tokens = 0, longest_tiled = 0;
+    for (const DecodeRow &r : rows) routed_tokens += r.len;
+    for (int b = 0; b < batch; b++)
+        if (!routed[b] && qo_indptr_host[b + 1] > qo_indptr_host[b]) longest_tiled = std::max<int64_t>(longest_tiled, kv_len[b]);
+    int layout = DSKV_LAYOUT_SEPARATE;
+    if (!rows.empty() && !tile_rows.empty()) {
+        const bool can_share = page_size >= 4;
+        if (route_one_row_requests == DSKV_ROUTE_SHARED_LAUNCH ||
+            (route_one_row_requests == DSKV_ROUTE_AUTO && routed_tokens >= kMinSharedLaunchTokens &&
+             longest_tiled >= kMinSharedLaunchTiledKeys))
+            layout = can_share ? DSKV_LAYOUT_SHARED : DSKV_LAYOUT_SEPARATE;
+        if (layout != DSKV_LAYOUT_SHARED && route_one_row_requests != DSKV_ROUTE_TWO_LAUNCHES) {
+            // not worth it, or not possible: everything as tiles
+            rows.clear();
+            std::fill(routed.begin(), routed.end(), 0);
+            tile_rows.clear();
+            for (int32_t r = 0; r < qo_indptr_host[batch]; r++) tile_rows.push_back(r);
+        }
+    }
+    info->layout = layout;
+    const int waves = layout == DSKV_LAYOUT_SHARED ? kPrefillWavesShared : kPrefillWaves;
     int64_t tile_words = 0;
     int rc = plan_tiles(qo_indptr_host, kv_len.data(), rows.empty() ? nullptr : routed.data(), batch,
                         n_qo_heads, n_kv_heads, head_dim, target_workgroups, plan_host, capacity_words,
-                        &info->n_tiles, &info->n_splits, &tile_words, &info->tile_workspace_bytes);
+                        &info->n_tiles, &info->n_splits, &tile_words, &info->tile_workspace_bytes, waves);
     if (rc) return rc;
     info->tile_workspace_bytes = (info->tile_workspace_bytes + 255) / 256 * 256;
     info->n_tile_rows = (int32_t)tile_rows.size();
@@ -957,7 +503,14 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     info->decode_plan_at = at;
     int64_t decode_words = 0;
     if (at > capacity_words) at = capacity_words;   // the decode planner then reports the shortage
-    rc = plan_decode_rows(rows.data(), (int32_t)rows.size(), n_qo_heads, head_dim, target_workgroups,
+    // shared launch: one decode workgroup (a share x a group of four kv heads) per compute unit
+    int32_t decode_target = target_workgroups;
+    if (layout == DSKV_LAYOUT_SHARED) {
+        const int head_groups = (n_kv_heads + kSharedWaves - 1) / kSharedWaves;
+        const int cus = target_workgroups > 0 ? std::min<int>(target_workgroups, kMaxWorkgroups) : compute_units();
+        decode_target = std::max(1, cus / head_groups);
+    }
+    rc = plan_decode_rows(rows.data(), (int32_t)rows.size(), n_qo_heads, head_dim, decode_target,
                           plan_host + at, capacity_words - at, &info->n_decode_items,
                           &info->n_decode_workgroups, &decode_words, &info->decode_workspace_bytes);
     if (rc) return rc;
@@ -978,6 +531,10 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
 }
 
 namespace dskv {
+
+static int launch_parts_merge(void *out, const float *part_o, const float *part_ml, const int32_t *rows,
+                              int32_t n_rows, int32_t n_splits, int32_t n_qo_heads, int32_t dtype,
+                              hipStream_t s);
 
 static bool prefill_mfma_path(int dtype, int head_dim, int n_qo_heads, int n_kv_heads, float scale_log2)
 {
@@ -1054,27 +611,9 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
         }
 #undef DSKV_LAUNCH_PREFILL
         DSKV_LAUNCH_CHECK("prefill_attn_mfma_kernel");
-        if (n_splits > 1) {   // the parts' partials become the output rows
-#define DSKV_LAUNCH_PARTS(DT, N)                                                                 \
-    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>),                                     \
-                       dim3((unsigned)(merge_rows ? n_merge_rows : nnz)), dim3(256), 0, s,      \
-                       (uint16_t *)out, part_o, part_ml, merge_rows, n_qo_heads)
-#define DSKV_LAUNCH_PARTS_N(DT)                                                  \
-    switch (n_splits) {                                                          \
-    case 2: DSKV_LAUNCH_PARTS(DT, 2); break;                                     \
-    case 3: DSKV_LAUNCH_PARTS(DT, 3); break;                                     \
-    case 4: DSKV_LAUNCH_PARTS(DT, 4); break;                                     \
-    case 5: DSKV_LAUNCH_PARTS(DT, 5); break;                                     \
-    case 6: DSKV_LAUNCH_PARTS(DT, 6); break;                                     \
-    case 7: DSKV_LAUNCH_PARTS(DT, 7); break;                                     \
-    default: DSKV_LAUNCH_PARTS(DT, 8); break;                                    \
-    }
-            if (dtype == DSKV_BF16) DSKV_LAUNCH_PARTS_N(DSKV_BF16)
-            else DSKV_LAUNCH_PARTS_N(DSKV_F16)
-#undef DSKV_LAUNCH_PARTS_N
-#undef DSKV_LAUNCH_PARTS
-            if (!merge_rows || n_merge_rows > 0) DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
-        }
+        if (n_splits > 1)   // the parts' partials become the output rows
+            return launch_parts_merge(out, part_o, part_ml, merge_rows, merge_rows ? n_merge_rows : nnz,
+                                      n_splits, n_qo_heads, dtype, s);
     } else {
         dim3 grid((unsigned)nnz, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_GEN(DT)                                                                      \
@@ -1087,6 +626,128 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
 #undef DSKV_LAUNCH_GEN
         DSKV_LAUNCH_CHECK("prefill_attn_generic_kernel");
     }
+    return 0;
+}
+
+// Merge pass of a tile plan in parts (see prefill_merge_parts_kernel).
+static int launch_parts_merge(void *out, const float *part_o, const float *part_ml, const int32_t *rows,
+                              int32_t n_rows, int32_t n_splits, int32_t n_qo_heads, int32_t dtype,
+                              hipStream_t s)
+{
+#define DSKV_LAUNCH_PARTS(DT, N)                                                                  \
+    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>), dim3((unsigned)n_rows), dim3(256), 0, s, \
+                       (uint16_t *)out, part_o, part_ml, rows, n_qo_heads)
+#define DSKV_LAUNCH_PARTS_N(DT)                                                  \
+    switch (n_splits) {                                                          \
+    case 2: DSKV_LAUNCH_PARTS(DT, 2); break;                                     \
+    case 3: DSKV_LAUNCH_PARTS(DT, 3); break;                                     \
+    case 4: DSKV_LAUNCH_PARTS(DT, 4); break;                                     \
+    case 5: DSKV_LAUNCH_PARTS(DT, 5); break;                                     \
+    case 6: DSKV_LAUNCH_PARTS(DT, 6); break;                                     \
+    case 7: DSKV_LAUNCH_PARTS(DT, 7); break;                                     \
+    default: DSKV_LAUNCH_PARTS(DT, 8); break;                                    \
+    }
+    if (dtype == DSKV_BF16) DSKV_LAUNCH_PARTS_N(DSKV_BF16)
+    else DSKV_LAUNCH_PARTS_N(DSKV_F16)
+#undef DSKV_LAUNCH_PARTS_N
+#undef DSKV_LAUNCH_PARTS
+    DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
+    return 0;
+}
+
+// One launch for a batch of decode rows and chunks (layout DSKV_LAYOUT_SHARED), then the two
+// merge passes.  The plan info comes from dskv_mixed_plan; everything in it that sizes a
+// launch or an array is checked here.
+static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indptr, const void *pages_layer,
+                               const int32_t *kv_page_indices, const int32_t *kv_page_indptr,
+                               const int32_t *kv_last_page_len, const int32_t *plan_dev,
+                               const dskv_mixed_plan_t *info, void *workspace, int64_t workspace_bytes,
+                               int32_t batch, int32_t nnz, int32_t n_qo_heads, int32_t n_kv_heads,
+                               int32_t head_dim, int32_t page_size, float sm_scale, int32_t causal,
+                               int32_t dtype, hipStream_t s)
+{
+    DSKV_REQUIRE(out && q && qo_indptr && pages_layer && kv_page_indices && kv_page_indptr && kv_last_page_len,
+                 "mixed_attn: null pointer argument");
+    DSKV_REQUIRE(decode_mfma_shape(head_dim, n_qo_heads, n_kv_heads, page_size) && page_size >= 4 &&
+                     (dtype == DSKV_BF16 || dtype == DSKV_F16),
+                 "mixed_attn: the shared launch takes 16-bit data, head_dim 128, groups up to 16 and "
+                 "power-of-two pages of at least 4 tokens");
+    DSKV_REQUIRE(((uintptr_t)out | (uintptr_t)q | (uintptr_t)pages_layer | (uintptr_t)workspace) % 16 == 0,
+                 "mixed_attn: out/q/pages/workspace must be 16-byte aligned");
+    DSKV_REQUIRE((int64_t)2 * page_size * n_kv_heads * head_dim * 2 < (int64_t(1) << 31),
+                 "mixed_attn: a page must be smaller than 2 GiB");
+    const int head_groups = (n_kv_heads + kSharedWaves - 1) / kSharedWaves;
+    const int32_t n_rows = info->n_decode_rows, n_items = info->n_decode_items, shares = info->n_decode_workgroups;
+    DSKV_REQUIRE(n_items >= n_rows && shares >= 1 && shares <= kMaxWorkgroups && info->n_tiles > 0 &&
+                     info->n_splits >= 1 && info->n_splits <= kMaxPrefillSplits && info->n_tiles % info->n_splits == 0,
+                 "mixed_attn: inconsistent plan (%d items of %d rows in %d shares, %d tile entries in %d parts)",
+                 n_items, n_rows, shares, info->n_tiles, info->n_splits);
+    const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
+    // workspace: partials of the tile parts, then those of cut decode rows
+    MixedArgs a{};
+    a.tile_max_slots = 0;
+    if (info->n_splits > 1) {
+        DSKV_REQUIRE(info->tile_workspace_bytes >= (int64_t)nnz * info->n_splits * slot_bytes,
+                     "mixed_attn: %d parts of %d rows need %lld bytes of partials, the plan reserves %lld",
+                     info->n_splits, nnz, (long long)((int64_t)nnz * info->n_splits * slot_bytes),
+                     (long long)info->tile_workspace_bytes);
+        a.tile_max_slots = (int)std::min<int64_t>(info->tile_workspace_bytes / slot_bytes, 1 << 30);
+        a.tile_part_o = reinterpret_cast<float *>(workspace);
+        a.tile_part_ml = a.tile_part_o + (int64_t)a.tile_max_slots * n_qo_heads * head_dim;
+    }
+    char *dec_ws = workspace ? (char *)workspace + info->tile_workspace_bytes : nullptr;
+    const int64_t dec_bytes = workspace ? workspace_bytes - info->tile_workspace_bytes : 0;
+    const int64_t dec_slots = std::min<int64_t>(dec_ws ? dec_bytes / slot_bytes : 0, 1 << 30);
+    DSKV_REQUIRE(n_items == n_rows || dec_slots >= (int64_t)n_items - n_rows + 1,
+                 "mixed_attn: workspace too small for %d decode items of %d rows", n_items, n_rows);
+    a.dec_max_slots = (int)dec_slots;
+    a.dec_part_o = reinterpret_cast<float *>(dec_ws);
+    a.dec_part_ml = a.dec_part_o ? a.dec_part_o + dec_slots * n_qo_heads * (int64_t)head_dim : nullptr;
+    const int32_t *dplan = plan_dev + info->decode_plan_at;
+    a.wg_ptr = dplan + kPlanHeaderWords;
+    const int32_t *req_parts = a.wg_ptr + shares + 1;
+    a.items = reinterpret_cast<const Item *>(req_parts + 2 * (int64_t)n_rows);
+    a.out = (uint16_t *)out;
+    a.q = (const uint16_t *)q;
+    a.pages = (const char *)pages_layer;
+    a.kv_indices = kv_page_indices;
+    a.n_qo_heads = n_qo_heads;
+    a.n_kv_heads = n_kv_heads;
+    a.page_shift = ilog2(page_size);
+    a.scale_log2 = sm_scale * 1.4426950408889634f;
+    DSKV_REQUIRE(a.scale_log2 > 1e-6f && a.scale_log2 < 1e6f, "mixed_attn: sm_scale out of range");
+    a.n_decode_wgs = shares * head_groups;
+    a.head_groups = head_groups;
+    a.qo_indptr = qo_indptr;
+    a.kv_indptr = kv_page_indptr;
+    a.kv_last = kv_last_page_len;
+    a.tile_info = plan_dev;
+    a.n_splits = info->n_splits;
+    a.causal = causal;
+    const int64_t grid = (int64_t)a.n_decode_wgs + (int64_t)info->n_tiles * n_kv_heads;
+    DSKV_REQUIRE(grid < (int64_t(1) << 31), "mixed_attn: too many workgroups");
+    const dim3 g((unsigned)grid), b(64 * kSharedWaves);
+#define DSKV_LAUNCH_MIXED(DT, PPT) hipLaunchKernelGGL((mixed_attn_kernel<DT, PPT>), g, b, 0, s, a)
+    if (dtype == DSKV_BF16) {
+        if (page_size >= kTile) DSKV_LAUNCH_MIXED(DSKV_BF16, 1);
+        else if (page_size == 8) DSKV_LAUNCH_MIXED(DSKV_BF16, 2);
+        else DSKV_LAUNCH_MIXED(DSKV_BF16, 0);
+    } else {
+        if (page_size >= kTile) DSKV_LAUNCH_MIXED(DSKV_F16, 1);
+        else if (page_size == 8) DSKV_LAUNCH_MIXED(DSKV_F16, 2);
+        else DSKV_LAUNCH_MIXED(DSKV_F16, 0);
+    }
+#undef DSKV_LAUNCH_MIXED
+    DSKV_LAUNCH_CHECK("mixed_attn_kernel");
+    if (n_items > n_rows) {
+        const bool wide = (int64_t)n_items > 32 * (int64_t)n_rows;
+        int rc = launch_partials_merge(out, a.dec_part_o, a.dec_part_ml, req_parts, plan_dev + info->row_map_at,
+                                       a.dec_max_slots, n_rows, n_qo_heads, head_dim, dtype, wide, s);
+        if (rc) return rc;
+    }
+    if (info->n_splits > 1)
+        return launch_parts_merge(out, a.tile_part_o, a.tile_part_ml, plan_dev + info->tile_rows_at,
+                                  info->n_tile_rows, info->n_splits, n_qo_heads, dtype, s);
     return 0;
 }
 
@@ -1141,6 +802,11 @@ extern "C" int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indpt
                  "mixed_attn: the plan needs a workspace of %lld bytes, got %lld",
                  (long long)(info->tile_workspace_bytes + info->decode_workspace_bytes),
                  (long long)workspace_bytes);
+    if (info->layout == DSKV_LAYOUT_SHARED)
+        return mixed_shared_launch(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
+                                   kv_last_page_len, plan_dev, info, workspace, workspace_bytes, batch, nnz,
+                                   n_qo_heads, n_kv_heads, head_dim, page_size, sm_scale, causal, dtype,
+                                   (hipStream_t)stream);
     // The one-row requests: the split-KV decode pass (each K/V byte read once, at the speed
     // of memory) and its merge; their partials lie behind those of the tile parts.
     int rc = decode_rows_attn(out, q, pages_layer, kv_page_indices, plan_dev + info->decode_plan_at,

@@ -349,8 +349,11 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         planned in several parts per tile, merged by a second pass, so that the launch has
         about this many workgroups (0: one per compute unit; negative: never split); the parts'
         partials go to the workspace buffer.
-        route_one_row_requests: False keeps one-row requests on the tile path (one live row
-        of a 64-row tile each), as for a plan of dskv_prefill_plan."""
+        route_one_row_requests: True lets the planner choose how one-row requests run (alone:
+        the decode kernel; beside chunks: one launch in which decode workgroups and query
+        tiles share the compute units, if the decode rows hold enough kv tokens); False keeps
+        them on the tile path (one live row of a 64-row tile each), as a plan of
+        dskv_prefill_plan does; _lib.ROUTE_TWO_LAUNCHES / _lib.ROUTE_SHARED_LAUNCH force a form."""
         self._shape_args(num_qo_heads, num_kv_heads, head_dim, page_size)
         self._qo_indptr, self._indptr = _i32(qo_indptr), _i32(paged_kv_indptr)
         self._indices, self._last = _i32(paged_kv_indices), _i32(paged_kv_last_page_len)
@@ -385,7 +388,8 @@ class BatchPrefillWithPagedKVCacheWrapper(_PagedWrapper):
         batch = h_qo.shape[0] - 1
         info = _lib.MixedPlanInfo()
         ws_bytes = self._workspace.numel() * self._workspace.element_size()
-        for target, routed in ((target_workgroups, route), (-1, route), (-1, False)):
+        route = int(route)          # True = _lib.ROUTE_AUTO
+        for target, routed in ((target_workgroups, route), (-1, route), (-1, _lib.ROUTE_OFF)):
             rc = _lib.lib().dskv_mixed_plan(h_qo.data_ptr(), h_kv.data_ptr(), h_last.data_ptr(), batch,
                                             self._p, self._hq, self._hkv, self._d, target, int(routed),
                                             plan.data_ptr(), cap, ctypes.byref(info))

@@ -249,17 +249,34 @@ int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const 
  * otherwise, and for a batch without one-row requests, plan and result are those of
  * dskv_prefill_plan / dskv_prefill_attn.  fp32 data is computed by the generic kernel,
  * whatever the plan routed.
+ * With DSKV_ROUTE_AUTO a batch of one-row requests only runs the decode pass alone; a batch
+ * of both kinds runs as ONE launch (DSKV_LAYOUT_SHARED: pages of at least 4 tokens, one-row
+ * requests holding at least 16384 kv tokens together, a tiled request of at least 4096 kv
+ * tokens) in which every compute unit hosts a decode workgroup, which keeps its memory path
+ * busy, and tile workgroups beside it, which use its matrix pipeline - or, where that launch
+ * does not apply or does not pay, as tiles only.  The two
+ * other modes force a layout (for measurements and tests).
  * The plan (at most dskv_mixed_plan_bound words; upload the first info->plan_words) holds
  * the tile entries, then at word decode_plan_at the decode work list, at row_map_at the
  * query row of every routed request and at tile_rows_at the rows the tiles cover.
  * workspace: tile_workspace_bytes (partials of tile parts) + decode_workspace_bytes
  * (partials of cut decode rows), 16-byte aligned.
  */
+/* route_one_row_requests */
+#define DSKV_ROUTE_OFF 0            /* every request as query tiles (the plan of dskv_prefill_plan) */
+#define DSKV_ROUTE_AUTO 1           /* the planner chooses (see dskv_mixed_plan) */
+#define DSKV_ROUTE_TWO_LAUNCHES 2   /* decode pass, then tile pass */
+#define DSKV_ROUTE_SHARED_LAUNCH 3  /* one launch whose decode and tile workgroups share the compute units */
+/* dskv_mixed_plan_t.layout */
+#define DSKV_LAYOUT_SEPARATE 0      /* tile pass and / or decode pass, workgroups of eight waves */
+#define DSKV_LAYOUT_SHARED 1        /* one launch of four-wave workgroups: a decode workgroup on every
+                                       compute unit, the tile workgroups beside them */
 typedef struct dskv_mixed_plan {
     int32_t n_tiles, n_splits;        /* tile entries (tiles x parts), parts per tile */
     int32_t n_tile_rows;              /* query rows computed by the tile pass */
     int32_t n_decode_rows;            /* one-row requests computed by the decode pass */
     int32_t n_decode_items, n_decode_workgroups;
+    int32_t layout, reserved;
     int64_t plan_words;
     int64_t decode_plan_at, row_map_at, tile_rows_at;
     int64_t tile_workspace_bytes, decode_workspace_bytes;

@@ -272,7 +272,8 @@ def _mixed_plan(lib, qo_lens, kv_lens, P=16, hq=32, hkv=8, d=128, target=0, rout
     return rc, info, plan, qo, indptr
 
 
-def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest():
+@pytest.mark.parametrize("mode", [_lib.ROUTE_AUTO, _lib.ROUTE_TWO_LAUNCHES, _lib.ROUTE_SHARED_LAUNCH])
+def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(mode):
     """The reference's mixed step (decode rows + one chunk through the prefill wrapper): every
     one-row request with kv tokens appears in the decode work list exactly once over its whole
     kv range, with its row of the ragged batch; every other row is covered by exactly one tile
@@ -280,21 +281,27 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest()
     lib = _lib.lib()
     rng = np.random.default_rng(5)
     qo_lens = [1] * 20 + [300] + [1] * 10 + [0, 1, 2]
-    kv_lens = list(rng.integers(200, 4000, size=20)) + [2500] + list(rng.integers(1, 50, size=10)) + [40, 0, 2]
-    rc, info, plan, qo, indptr = _mixed_plan(lib, qo_lens, kv_lens)
+    kv_lens = list(rng.integers(200, 4000, size=20)) + [4500] + list(rng.integers(1, 50, size=10)) + [40, 0, 2]
+    rc, info, plan, qo, indptr = _mixed_plan(lib, qo_lens, kv_lens, route=mode)
     assert rc == 0, _lib.last_error()
+    # 30 decode rows with more than 16384 kv tokens beside tiles: one shared launch unless told otherwise
+    shared = mode != _lib.ROUTE_TWO_LAUNCHES
+    assert info.layout == (_lib.LAYOUT_SHARED if shared else _lib.LAYOUT_SEPARATE)
     routed = [b for b in range(len(qo_lens)) if qo_lens[b] == 1 and kv_lens[b] > 0]
     assert info.n_decode_rows == len(routed) == 30 and info.n_tile_rows == 300 + 1 + 2
     assert info.n_decode_rows + info.n_tile_rows == int(qo[-1])
     # tiles: only requests 20 (300 rows), 32 (one row without kv tokens) and 33 (two rows)
     tiles = plan[: 5 * info.n_tiles].reshape(-1, 5)
     assert sorted(set(tiles[:, 0].tolist())) == [20, 32, 33]
-    assert info.n_tiles == (5 + 1 + 1) * info.n_splits
+    # tiles of 64 query rows (eight waves), or of 32 in the launch of four-wave workgroups
+    assert info.n_tiles == ((10 if shared else 5) + 1 + 1) * info.n_splits
     assert info.decode_plan_at % 4 == 0 and info.decode_plan_at >= 5 * info.n_tiles
     # the decode work list has dskv_decode_plan's layout; its items name ragged rows
     dp = plan[info.decode_plan_at:]
     n_items, wgs, n_slots, batch = dp[:4].tolist()
     assert (n_items, wgs, batch) == (info.n_decode_items, info.n_decode_workgroups, info.n_decode_rows)
+    if shared:          # one decode workgroup (a share x 4 of the 8 kv heads) per compute unit, 256 without a GPU
+        assert wgs == 128
     items = dp[4 + wgs + 1 + 2 * batch: 4 + wgs + 1 + 2 * batch + 8 * n_items].reshape(-1, 8)
     assert info.row_map_at == info.decode_plan_at + 4 + wgs + 1 + 2 * batch + 8 * n_items
     row_map = plan[info.row_map_at: info.row_map_at + batch]
@@ -331,13 +338,26 @@ def test_mixed_plan_without_routing_is_the_prefill_plan():
         assert info.n_tile_rows == 203 and info.n_splits == splits_k
         assert plan[: info.plan_words].tolist() == want_k.reshape(-1).tolist()
         assert info.tile_workspace_bytes == -(-ws_k // 256) * 256
-    # a batch of decode rows only (the reference's benchmark/mixed.py without a chunk): no tiles
-    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 1], [700, 33, 16])
-    assert rc == 0 and info.n_tiles == 0 and info.n_tile_rows == 0 and info.n_decode_rows == 3
-    assert info.decode_plan_at == 0
+    # a batch of decode rows only (the reference's benchmark/mixed.py without a chunk): no tiles,
+    # the decode kernel by itself in every routing mode
+    for mode in (_lib.ROUTE_AUTO, _lib.ROUTE_TWO_LAUNCHES, _lib.ROUTE_SHARED_LAUNCH):
+        rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 1], [700, 33, 16], route=mode)
+        assert rc == 0 and info.n_tiles == 0 and info.n_tile_rows == 0 and info.n_decode_rows == 3
+        assert info.decode_plan_at == 0 and info.layout == _lib.LAYOUT_SEPARATE
+    # few kv tokens behind the one-row requests of a batch with chunks: all tiles, unless forced
+    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 200], [700, 33, 900])
+    assert rc == 0 and info.n_decode_rows == 0 and info.n_tile_rows == 202 and info.layout == _lib.LAYOUT_SEPARATE
+    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 200], [700, 33, 900], route=_lib.ROUTE_SHARED_LAUNCH)
+    assert rc == 0 and info.n_decode_rows == 2 and info.n_tile_rows == 200 and info.layout == _lib.LAYOUT_SHARED
+    # pages of two tokens: no shared launch; forced, the batch is planned as tiles
+    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 200], [700, 33, 900], P=2, route=_lib.ROUTE_SHARED_LAUNCH)
+    assert rc == 0 and info.n_decode_rows == 0 and info.layout == _lib.LAYOUT_SEPARATE
+    rc, info, plan, _, _ = _mixed_plan(lib, [1, 1, 200], [700, 33, 900], P=2, route=_lib.ROUTE_TWO_LAUNCHES)
+    assert rc == 0 and info.n_decode_rows == 2 and info.layout == _lib.LAYOUT_SEPARATE
+    assert _mixed_plan(lib, [1, 5], [700, 33], route=4)[0] == -1
     # refusals
     assert _mixed_plan(lib, [1, 5], [700, 33], cap=6)[0] == -2
-    assert _mixed_plan(lib, [1, 200], [700, 900], cap=5 * 4 + 8)[0] == -2
+    assert _mixed_plan(lib, [1, 200], [700, 900], cap=5 * 4 + 8, route=_lib.ROUTE_TWO_LAUNCHES)[0] == -2
     assert _mixed_plan(lib, [1, 5], [700, 33], hq=30)[0] == -1
     assert lib.dskv_mixed_plan(None, None, None, 0, 16, 32, 8, 128, 0, 1, None, 0, None) == -1
     info = _lib.MixedPlanInfo()

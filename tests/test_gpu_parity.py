@@ -482,7 +482,7 @@ MIXED_CASES = [
     ("page2_mha", [50, 37, 64], [1, 20, 1], 2, 8, 8, "bf16", 0, 2),
     ("f32_generic_kernel", [100, 37, 64], [1, 20, 1], 16, 32, 8, "f32", 0, 2),
     ("group32_stays_tiled", [100, 37, 64], [1, 20, 1], 16, 32, 1, "bf16", 0, 0),
-    ("many_rows", [17 * i % 900 + 1 for i in range(75)] + [2500], [1] * 75 + [437], 16, 32, 8, "bf16", 0, 75),
+    ("many_rows", [17 * i % 900 + 1 for i in range(75)] + [4500], [1] * 75 + [437], 16, 32, 8, "bf16", 0, 75),
 ]
 
 
@@ -499,13 +499,28 @@ def test_mixed_batch_routes_one_row_requests_to_the_decode_kernel(case):
     _announce("mixed", name, P, Hq, Hkv, dtype, target)
     sc = make_scenario(43, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
     w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(96 << 20, dtype=torch.uint8, device="cuda"))
+    from deserve_amd import _lib
+
     q, pages = to_torch(sc.q, dtype), to_torch(sc.pages, dtype)
-    for route in (True, False):
+    tiled_rows = sum(n for n, k in zip(qo, kv) if n != 1 or k == 0)
+    for route in (_lib.ROUTE_SHARED_LAUNCH, _lib.ROUTE_TWO_LAUNCHES, True, False):
         w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
                         _dev_i32(sc.kv_last_page_lens), Hq, Hkv, 128, P, target_workgroups=target,
                         route_one_row_requests=route)
-        assert w._n_decode_rows == (n_routed if route else 0)
-        if name == "cut_rows" and route:
+        shared = w._info.layout == _lib.LAYOUT_SHARED
+        if route == _lib.ROUTE_SHARED_LAUNCH:
+            # one launch for both kinds of rows wherever there are both and pages hold >= 4 tokens
+            assert shared == (n_routed > 0 and tiled_rows > 0 and P >= 4), name
+            assert w._n_decode_rows == (n_routed if shared or tiled_rows == 0 else 0)
+        elif route == _lib.ROUTE_TWO_LAUNCHES:
+            assert not shared and w._n_decode_rows == n_routed
+        elif route is True:
+            assert w._n_decode_rows in (0, n_routed)
+            if name == "many_rows":
+                assert shared and w._n_decode_rows == 75              # the planner's own choice for such a step
+        else:
+            assert not shared and w._n_decode_rows == 0
+        if name == "cut_rows" and route in (_lib.ROUTE_SHARED_LAUNCH, _lib.ROUTE_TWO_LAUNCHES):
             assert w._info.n_decode_items > w._n_decode_rows          # rows cut across workgroups: merged
         for causal in (True, False):
             out = torch.full_like(q, float("nan"))
@@ -515,7 +530,7 @@ def test_mixed_batch_routes_one_row_requests_to_the_decode_kernel(case):
             want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices,
                                          sc.kv_page_indptr, sc.kv_last_page_lens, dtype, causal=causal)
             assert np.isfinite(got).all(), (name, route, causal)
-            assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (name, route, causal)
+            assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (name, route, causal, w._info.layout)
         w.end_forward()
 
 
