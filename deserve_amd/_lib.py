@@ -26,7 +26,7 @@ class MixedPlanInfo(ctypes.Structure):
     _fields_ = [("n_tiles", c_int32), ("n_splits", c_int32), ("n_tile_rows", c_int32),
                 ("n_decode_rows", c_int32), ("n_decode_items", c_int32), ("n_decode_workgroups", c_int32),
                 ("layout", c_int32), ("reserved", c_int32), ("plan_words", c_int64), ("decode_plan_at", c_int64), ("row_map_at", c_int64),
-                ("tile_rows_at", c_int64), ("tile_workspace_bytes", c_int64),
+                ("tile_workspace_bytes", c_int64),
                 ("decode_workspace_bytes", c_int64)]
 
 

@@ -133,28 +133,26 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
     }
 }
 
-// Merge pass of a plan in parts: output row r, head qh = sum_i w_i O_i / sum_i w_i l_i over
-// the n_splits partials of the row (slots r * n_splits + i), w_i = exp2(m_i - max_j m_j).
-// One workgroup per query row; a thread owns 16 consecutive dims of one head and requests
-// all of its parts' values at once (no block table, no lookup: the slots follow from the
-// row).  The decode path's merge kernel, launched with one wave per (row, head) and a table
-// of parts per row, took 11.5 us for the 512 rows of a chunk; this one takes about half.
+// Merge pass of a plan with tiles in parts: output row r, head qh = sum_i w_i O_i / sum_i w_i l_i
+// over the row's partials, w_i = exp2(m_i - max_j m_j).  row_parts[2 r] = the row's first slot,
+// row_parts[2 r + 1] = its number of parts (consecutive slots); 0: the row was written by its
+// tile (or by the decode kernel) and is left alone.  One workgroup per query row; a thread
+// owns 16 consecutive dims of one head and requests all of its parts' values at once.  The
+// decode path's merge kernel, launched with one wave per (row, head), took 11.5 us for the
+// 512 rows of a chunk; this one takes about half.
 template <int DT, int kParts>
-__global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
-    uint16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
-    const int32_t *__restrict__ rows, int n_qo_heads)
+__device__ __forceinline__ void merge_row_parts(uint16_t *__restrict__ out, const float *__restrict__ part_o,
+                                                const float *__restrict__ part_ml, long row, long first,
+                                                int n_qo_heads)
 {
     typedef Elt<DT> E;
-    // rows (may be null): the query rows that were computed in parts, when they are not all
-    // rows of the batch (the others were left to the decode kernel)
-    const long row = rows ? rows[blockIdx.x] : blockIdx.x;
     for (int idx = threadIdx.x; idx < n_qo_heads * (kHeadDim / 16); idx += blockDim.x) {
         const int qh = idx / (kHeadDim / 16), d0 = (idx % (kHeadDim / 16)) * 16;
         f32x4 o[kParts][4];
         float m[kParts], l[kParts];
 #pragma unroll
         for (int i = 0; i < kParts; i++) {
-            const long slot = row * kParts + i;
+            const long slot = first + i;
             const float *src = part_o + (slot * n_qo_heads + qh) * kHeadDim + d0;
 #pragma unroll
             for (int j = 0; j < 4; j++) o[i][j] = *reinterpret_cast<const f32x4 *>(src + 4 * j);
@@ -184,6 +182,28 @@ __global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
                               E::pack2(acc[j + 1][2] * inv, acc[j + 1][3] * inv)};
             *reinterpret_cast<u32x4 *>(dst + 4 * j) = w4;
         }
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
+    uint16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
+    const int32_t *__restrict__ row_parts, int max_slots, int n_qo_heads)
+{
+    const long row = blockIdx.x;
+    const const_i32_ptr table = as_const(row_parts) + 2 * row;
+    const int first = table[0], n = table[1];   // uniform over the workgroup
+    if (n <= 0 || first < 0 || first + n > max_slots) return;
+    switch (n) {
+    case 1: merge_row_parts<DT, 1>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 2: merge_row_parts<DT, 2>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 3: merge_row_parts<DT, 3>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 4: merge_row_parts<DT, 4>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 5: merge_row_parts<DT, 5>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 6: merge_row_parts<DT, 6>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 7: merge_row_parts<DT, 7>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    case 8: merge_row_parts<DT, 8>(out, part_o, part_ml, row, first, n_qo_heads); break;
+    default: break;   // the planner never cuts a tile into more parts
     }
 }
 
@@ -234,7 +254,7 @@ struct MixedArgs {
     // tile side
     const int32_t *qo_indptr, *kv_indptr, *kv_last, *tile_info;
     float *tile_part_o, *tile_part_ml;
-    int tile_max_slots, n_splits, causal;
+    int tile_max_slots, causal;
 };
 
 template <int DT, int kPagesPerTile>
@@ -253,7 +273,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, 2) void mixed_attn_kernel(const 
         __builtin_amdgcn_s_setprio(kSharedTilePriority);
         prefill_attn_body<DT, true, kPrefillWavesShared>(
             lds, wg - a.n_decode_wgs, a.out, a.q, a.qo_indptr, a.pages, a.kv_indices, a.kv_indptr, a.kv_last,
-            a.tile_info, a.n_qo_heads, a.n_kv_heads, a.page_shift, a.scale_log2, a.causal, a.n_splits,
+            a.tile_info, a.n_qo_heads, a.n_kv_heads, a.page_shift, a.scale_log2, a.causal,
             a.tile_part_o, a.tile_part_ml, a.tile_max_slots);
     }
 }
@@ -268,6 +288,8 @@ constexpr int kMaxPrefillSplits = 8;         // parts a tile's K/V range is cut 
 // context lost a fifth of what the parts buy
 constexpr int kMinSplitTokens = 512;
 constexpr int kMaxSplitTarget = 1024;        // workgroups a split plan aims at, at most
+// a workgroup's start and end, in 32-token blocks of walking (for the fair share of a launch)
+constexpr int kTileOverheadBlocks = 4;
 constexpr int32_t kWholeRange = 0x7fffffff;  // blk_end of a tile that is not split
 // kv tokens the one-row requests of a mixed batch must hold together before they get decode
 // workgroups of their own beside the tiles (64 MB of K/V per layer in the 8-kv-head bf16 shape)
@@ -291,24 +313,27 @@ extern "C" int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz)
 {
     using namespace dskv;
     if (batch < 0 || nnz < 0) return 0;
-    // entries: one per tile, or per part of a tile when the plan splits (then there are few
-    // tiles: at most 2 * kMaxSplitTarget parts)
-    return kTileWords * ((int64_t)batch + nnz + 2 * kMaxSplitTarget);
+    // entries: one per tile (at most batch + nnz of them), times the parts of those that are
+    // cut: filling the chip adds at most 2 * kMaxSplitTarget entries, cutting long walks down
+    // to the fair share at most 2 * kMaxSplitTarget more; then two words per query row
+    return kTileWords * ((int64_t)batch + nnz + 4 * kMaxSplitTarget + kMaxPrefillSplits) + 2 * nnz;
 }
 
 namespace dskv {
 
 // The tile planner.  skip (may be null): requests marked there get no tiles (their single
-// row is computed by the decode kernel).
+// row is computed by the decode kernel).  Plan: the tile entries (kTileWords each), then, if
+// any tile is cut into parts, two words per query row of the batch (first partial slot,
+// number of parts; 0 parts = the row needs no merge).
 static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host, const char *skip,
                       int32_t batch, int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
                       int32_t target_workgroups, int32_t *plan_host, int64_t capacity_words,
                       int32_t *n_tiles_out, int32_t *n_splits_out, int64_t *plan_words_out,
-                      int64_t *workspace_bytes_out, int waves = kPrefillWaves)
+                      int64_t *workspace_bytes_out, int waves = kPrefillWaves, bool cut_long_walks = true)
 {
     const int rows = prefill_rows_per_tile(n_qo_heads, n_kv_heads, waves);
     // later query tiles of a request see more keys: they come first within a request
-    struct Tile { int32_t b, row; int64_t keys; };
+    struct Tile { int32_t b, row, n_rows, parts; int64_t keys, first_slot; };
     std::vector<Tile> tiles;
     int64_t nnz = 0;
     for (int b = 0; b < batch; b++) {
@@ -319,7 +344,7 @@ static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
         for (int64_t i = (n_b + rows - 1) / rows - 1; i >= 0; i--) {
             const int64_t last_row = std::min<int64_t>(i * rows + rows, n_b) - 1;
             const int64_t keys = kv_len_host ? std::max<int64_t>((int64_t)kv_len_host[b] - n_b + last_row + 1, 0) : 0;
-            tiles.push_back({b, (int32_t)(i * rows), keys});
+            tiles.push_back({b, (int32_t)(i * rows), (int32_t)(last_row + 1 - i * rows), 1, keys, 0});
         }
     }
     DSKV_REQUIRE(tiles.size() < (size_t(1) << 26) && nnz < (int64_t(1) << 31), "prefill_plan: too many tiles");
@@ -329,29 +354,65 @@ static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
     if (kv_len_host && tiles.size() > 1)
         std::stable_sort(tiles.begin(), tiles.end(),
                          [](const Tile &x, const Tile &y) { return x.keys > y.keys; });
-    // Few tiles (a chunk of a few hundred tokens, as the reference's scheduler hands out:
-    // one 512-token chunk of an 8-kv-head model is 64 workgroups) leave most of the chip
-    // idle: then every tile's K/V range is cut into parts that run as workgroups of their
-    // own and leave partials, merged by a second pass - the decode path's way of keeping
-    // all compute units busy.  Needs the kv lengths and the 16-bit kernel's head dim.
-    int splits = 1;
+    // Parts.  A tile's K/V range can be cut into parts that run as workgroups of their own and
+    // leave partials, merged by a second pass - the decode path's way of keeping all compute
+    // units busy.  Needs the kv lengths and the 16-bit kernel's head dim.  Two reasons to cut:
+    //  * few tiles (a chunk of a few hundred tokens, as the reference's scheduler hands out:
+    //    one 512-token chunk of an 8-kv-head model is 64 workgroups) leave most of the chip
+    //    idle: every tile is cut into as many parts as fill it;
+    //  * a tile whose walk is longer than the launch's fair share per compute unit ends the
+    //    launch by itself (a chunk behind 8000 tokens in a step of decode rows: 232 us, with
+    //    its tiles cut in two 197 us): it is cut down to that share.  Cutting further does
+    //    not pay: with walks of at most half (a quarter of) the share a mixed step of 75
+    //    decode rows and a chunk takes 159 (178) us instead of 149 us - the partials cost more
+    //    than the shorter tail buys.  For the same reason only outliers are cut: when the
+    //    tiles above the share hold more than a quarter of the launch's blocks (one long
+    //    prompt of many tiles, the later ones longer), the launch is made of them, every cut
+    //    tile would pay for partials, and the longest-first order is left to do its work.
+    int max_parts = 1;
     if (kv_len_host && head_dim == kHeadDim && target_workgroups >= 0 && !tiles.empty()) {
         const int64_t target =
             target_workgroups > 0 ? std::min<int64_t>(target_workgroups, kMaxSplitTarget) : compute_units();
         const int64_t wgs = (int64_t)tiles.size() * n_kv_heads;
-        if (wgs * 2 <= target) {
-            splits = (int)std::min<int64_t>(kMaxPrefillSplits, target / wgs);
-            splits = (int)std::min<int64_t>(splits, std::max<int64_t>(1, tiles.front().keys / kMinSplitTokens));
+        int fill = 1;
+        if (wgs * 2 <= target) fill = (int)std::min<int64_t>(kMaxPrefillSplits, target / wgs);
+        int64_t total_blocks = 0;
+        for (const Tile &t : tiles) total_blocks += (t.keys + kBlock - 1) / kBlock + kTileOverheadBlocks;
+        // blocks one compute unit walks if the launch is shared out evenly, and the longest
+        // walk a single workgroup may then have
+        const int64_t share = (total_blocks * n_kv_heads + target - 1) / target;
+        const int64_t cap = std::max<int64_t>(kMinSplitTokens / kBlock, share);
+        int64_t above = 0;
+        for (const Tile &t : tiles)
+            if ((t.keys + kBlock - 1) / kBlock > cap) above += (t.keys + kBlock - 1) / kBlock;
+        if (above * 4 > total_blocks) cut_long_walks = false;
+        for (Tile &t : tiles) {
+            const int64_t blocks = (t.keys + kBlock - 1) / kBlock;
+            int64_t parts = std::max<int64_t>(fill, cut_long_walks ? (blocks + cap - 1) / cap : 1);
+            parts = std::min<int64_t>(parts, kMaxPrefillSplits);
+            parts = std::min<int64_t>(parts, std::max<int64_t>(1, t.keys / kMinSplitTokens));
+            t.parts = (int32_t)parts;
+            max_parts = std::max(max_parts, t.parts);
         }
     }
-    const int64_t n_entries = (int64_t)tiles.size() * splits;
-    const int64_t words = n_entries * kTileWords;
+    int64_t n_entries = 0, n_slots = 0;
+    for (Tile &t : tiles) {
+        n_entries += t.parts;
+        if (t.parts > 1) {
+            t.first_slot = n_slots;
+            n_slots += (int64_t)t.n_rows * t.parts;
+        }
+    }
+    DSKV_REQUIRE(n_slots < (int64_t(1) << 31), "prefill_plan: too many partial slots");
+    const int64_t words = n_entries * kTileWords + (max_parts > 1 ? 2 * nnz : 0);
     if (words > capacity_words) {
         set_error("prefill_plan: plan needs %lld words, buffer has %lld", (long long)words,
                   (long long)capacity_words);
         return DSKV_E_NOMEM;
     }
     int32_t *p = plan_host;
+    int32_t *row_parts = plan_host + n_entries * kTileWords;
+    if (max_parts > 1) std::fill(row_parts, row_parts + 2 * nnz, 0);
     for (const Tile &t : tiles) {
         // Parts of equal length, in units of four 32-token blocks (the kernel's loop is
         // unrolled by four), measured on the keys the tile sees under the causal mask; the
@@ -359,20 +420,26 @@ static int plan_tiles(const int32_t *qo_indptr_host, const int32_t *kv_len_host,
         // also right without the mask (the last part then holds the rest of the request); a
         // part that starts past what the tile sees is empty.
         const int64_t blocks = (t.keys + kBlock - 1) / kBlock;
-        const int64_t chunk = ((blocks + splits - 1) / splits + 3) / 4 * 4;
-        for (int s = 0; s < splits; s++) {
+        const int64_t chunk = ((blocks + t.parts - 1) / t.parts + 3) / 4 * 4;
+        for (int s = 0; s < t.parts; s++) {
             *p++ = t.b;
             *p++ = t.row;
             *p++ = (int32_t)(s * chunk);
-            *p++ = s + 1 < splits ? (int32_t)((s + 1) * chunk) : kWholeRange;
-            *p++ = s;
+            *p++ = s + 1 < t.parts ? (int32_t)((s + 1) * chunk) : kWholeRange;
+            *p++ = t.parts > 1 ? (s | (t.parts << 8)) : -1;
+            *p++ = (int32_t)t.first_slot;
         }
+        if (t.parts > 1)
+            for (int r = 0; r < t.n_rows; r++) {
+                const int64_t row = (int64_t)qo_indptr_host[t.b] + t.row + r;
+                row_parts[2 * row] = (int32_t)(t.first_slot + (int64_t)r * t.parts);
+                row_parts[2 * row + 1] = t.parts;
+            }
     }
     *n_tiles_out = (int32_t)n_entries;
-    *n_splits_out = splits;
+    *n_splits_out = max_parts;
     *plan_words_out = words;
-    *workspace_bytes_out =
-        splits > 1 ? nnz * splits * (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float) : 0;
+    *workspace_bytes_out = n_slots * (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
     return 0;
 }
 
@@ -441,7 +508,7 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     std::vector<int32_t> kv_len(batch);
     std::vector<char> routed(batch, 0);
     std::vector<DecodeRow> rows;
-    std::vector<int32_t> tile_rows;
+    int64_t n_tile_rows = 0;
     for (int b = 0; b < batch; b++) {
         const int64_t np = (int64_t)kv_page_indptr_host[b + 1] - kv_page_indptr_host[b];
         DSKV_REQUIRE(np >= 0, "mixed_plan: kv_page_indptr not monotone at %d", b);
@@ -457,7 +524,7 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
             routed[b] = 1;
             rows.push_back(DecodeRow{len, kv_page_indptr_host[b], qo_indptr_host[b]});
         } else {
-            for (int64_t i = 0; i < n_b; i++) tile_rows.push_back((int32_t)(qo_indptr_host[b] + i));
+            n_tile_rows += n_b;
         }
     }
     // How the routed rows run.  Without tiled rows: the decode kernel by itself (workgroups of
@@ -474,7 +541,7 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     for (int b = 0; b < batch; b++)
         if (!routed[b] && qo_indptr_host[b + 1] > qo_indptr_host[b]) longest_tiled = std::max<int64_t>(longest_tiled, kv_len[b]);
     int layout = DSKV_LAYOUT_SEPARATE;
-    if (!rows.empty() && !tile_rows.empty()) {
+    if (!rows.empty() && n_tile_rows > 0) {
         const bool can_share = page_size >= 4;
         if (route_one_row_requests == DSKV_ROUTE_SHARED_LAUNCH ||
             (route_one_row_requests == DSKV_ROUTE_AUTO && routed_tokens >= kMinSharedLaunchTokens &&
@@ -484,8 +551,7 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
             // not worth it, or not possible: everything as tiles
             rows.clear();
             std::fill(routed.begin(), routed.end(), 0);
-            tile_rows.clear();
-            for (int32_t r = 0; r < qo_indptr_host[batch]; r++) tile_rows.push_back(r);
+            n_tile_rows = qo_indptr_host[batch];
         }
     }
     info->layout = layout;
@@ -493,10 +559,12 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     int64_t tile_words = 0;
     int rc = plan_tiles(qo_indptr_host, kv_len.data(), rows.empty() ? nullptr : routed.data(), batch,
                         n_qo_heads, n_kv_heads, head_dim, target_workgroups, plan_host, capacity_words,
-                        &info->n_tiles, &info->n_splits, &tile_words, &info->tile_workspace_bytes, waves);
+                        &info->n_tiles, &info->n_splits, &tile_words, &info->tile_workspace_bytes, waves,
+                        /* the tiles of a shared launch run beside decode workgroups for its whole length */
+                        layout != DSKV_LAYOUT_SHARED);
     if (rc) return rc;
     info->tile_workspace_bytes = (info->tile_workspace_bytes + 255) / 256 * 256;
-    info->n_tile_rows = (int32_t)tile_rows.size();
+    info->n_tile_rows = (int32_t)n_tile_rows;
     int64_t at = (tile_words + 3) / 4 * 4;
     info->plan_words = tile_words;
     if (rows.empty()) return 0;
@@ -516,7 +584,7 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     if (rc) return rc;
     info->n_decode_rows = (int32_t)rows.size();
     at += decode_words;
-    const int64_t total = at + (int64_t)rows.size() + (int64_t)tile_rows.size();
+    const int64_t total = at + (int64_t)rows.size();
     if (total > capacity_words) {
         set_error("mixed_plan: plan needs %lld words, buffer has %lld", (long long)total,
                   (long long)capacity_words);
@@ -524,17 +592,15 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     }
     info->row_map_at = at;
     for (const DecodeRow &r : rows) plan_host[at++] = r.row;
-    info->tile_rows_at = at;
-    std::copy(tile_rows.begin(), tile_rows.end(), plan_host + at);
     info->plan_words = total;
     return 0;
 }
 
 namespace dskv {
 
-static int launch_parts_merge(void *out, const float *part_o, const float *part_ml, const int32_t *rows,
-                              int32_t n_rows, int32_t n_splits, int32_t n_qo_heads, int32_t dtype,
-                              hipStream_t s);
+static int launch_parts_merge(void *out, const float *part_o, const float *part_ml,
+                              const int32_t *row_parts, int32_t nnz, int64_t max_slots,
+                              int32_t n_qo_heads, int32_t dtype, hipStream_t s);
 
 static bool prefill_mfma_path(int dtype, int head_dim, int n_qo_heads, int n_kv_heads, float scale_log2)
 {
@@ -543,8 +609,8 @@ static bool prefill_mfma_path(int dtype, int head_dim, int n_qo_heads, int n_kv_
            n_qo_heads / n_kv_heads <= kWaveCols && scale_log2 > 1e-6f && scale_log2 < 1e6f;
 }
 
-// merge_rows / n_merge_rows: the query rows the tiles cover when they are not all nnz rows of
-// the batch (null: all of them); an MFMA-path call with n_tiles == 0 then has nothing to do.
+// some_rows_elsewhere: the tiles do not cover all nnz rows of the batch (the others are the
+// decode kernel's); an MFMA-path call with n_tiles == 0 then has nothing to do.
 static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
                              const void *pages_layer, const int32_t *kv_page_indices,
                              const int32_t *kv_page_indptr, const int32_t *kv_last_page_len,
@@ -552,7 +618,7 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
                              void *workspace, int64_t workspace_bytes, int32_t batch, int32_t nnz,
                              int32_t n_qo_heads, int32_t n_kv_heads, int32_t head_dim,
                              int32_t page_size, float sm_scale, int32_t causal, int32_t dtype,
-                             void *stream, const int32_t *merge_rows, int32_t n_merge_rows)
+                             void *stream, bool some_rows_elsewhere)
 {
     DSKV_REQUIRE(batch >= 0 && nnz >= 0 && n_tiles >= 0, "prefill_attn: negative sizes");
     if (batch == 0 || nnz == 0) return 0;
@@ -571,19 +637,20 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
     const float scale_log2 = sm_scale * 1.4426950408889634f;
     hipStream_t s = (hipStream_t)stream;
     const bool mfma = prefill_mfma_path(dtype, head_dim, n_qo_heads, n_kv_heads, scale_log2);
-    if (mfma && merge_rows && n_tiles == 0) return 0;   // every row went to the decode kernel
+    if (mfma && some_rows_elsewhere && n_tiles == 0) return 0;   // every row went to the decode kernel
     if (mfma) {
         DSKV_REQUIRE(plan_dev && n_tiles > 0, "prefill_attn: missing plan");
-        DSKV_REQUIRE(n_splits >= 1 && n_splits <= kMaxPrefillSplits && n_tiles % n_splits == 0,
-                     "prefill_attn: %d plan entries in %d parts", n_tiles, n_splits);
+        DSKV_REQUIRE(n_splits >= 1 && n_splits <= kMaxPrefillSplits,
+                     "prefill_attn: tiles in up to %d parts", n_splits);
         float *part_o = nullptr, *part_ml = nullptr;
         int64_t max_slots = 0;
         if (n_splits > 1) {
+            // the plan's partial slots are numbered from 0; the kernels never touch a slot at or
+            // beyond max_slots, so a workspace smaller than the plan asked for loses rows, not memory
             const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
-            DSKV_REQUIRE(workspace && workspace_bytes >= (int64_t)nnz * n_splits * slot_bytes &&
-                             (uintptr_t)workspace % 16 == 0,
-                         "prefill_attn: a plan in %d parts needs a 16-byte aligned workspace of %lld bytes, got %lld",
-                         n_splits, (long long)((int64_t)nnz * n_splits * slot_bytes), (long long)workspace_bytes);
+            DSKV_REQUIRE(workspace && workspace_bytes >= slot_bytes && (uintptr_t)workspace % 16 == 0,
+                         "prefill_attn: a plan with tiles in parts needs a 16-byte aligned workspace "
+                         "(dskv_prefill_plan says how large), got %lld bytes", (long long)workspace_bytes);
             max_slots = std::min<int64_t>(workspace_bytes / slot_bytes, 1 << 30);
             part_o = reinterpret_cast<float *>(workspace);
             part_ml = part_o + max_slots * n_qo_heads * (int64_t)head_dim;
@@ -600,8 +667,8 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
     hipLaunchKernelGGL((prefill_attn_mfma_kernel<DT, SHARE>), grid, block, 0, s, (uint16_t *)out, \
                        (const uint16_t *)q, qo_indptr, (const char *)pages_layer,               \
                        kv_page_indices, kv_page_indptr, kv_last_page_len, plan_dev,             \
-                       n_qo_heads, n_kv_heads, shift, scale_log2, causal, n_splits, part_o,     \
-                       part_ml, (int)max_slots)
+                       n_qo_heads, n_kv_heads, shift, scale_log2, causal, part_o, part_ml,     \
+                       (int)max_slots)
         if (dtype == DSKV_BF16) {
             if (page_size >= 4) DSKV_LAUNCH_PREFILL(DSKV_BF16, true);
             else DSKV_LAUNCH_PREFILL(DSKV_BF16, false);
@@ -612,8 +679,8 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
 #undef DSKV_LAUNCH_PREFILL
         DSKV_LAUNCH_CHECK("prefill_attn_mfma_kernel");
         if (n_splits > 1)   // the parts' partials become the output rows
-            return launch_parts_merge(out, part_o, part_ml, merge_rows, merge_rows ? n_merge_rows : nnz,
-                                      n_splits, n_qo_heads, dtype, s);
+            return launch_parts_merge(out, part_o, part_ml, plan_dev + (int64_t)n_tiles * kTileWords, nnz,
+                                      max_slots, n_qo_heads, dtype, s);
     } else {
         dim3 grid((unsigned)nnz, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_GEN(DT)                                                                      \
@@ -629,28 +696,18 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
     return 0;
 }
 
-// Merge pass of a tile plan in parts (see prefill_merge_parts_kernel).
-static int launch_parts_merge(void *out, const float *part_o, const float *part_ml, const int32_t *rows,
-                              int32_t n_rows, int32_t n_splits, int32_t n_qo_heads, int32_t dtype,
-                              hipStream_t s)
+// Merge pass of a tile plan with parts (see prefill_merge_parts_kernel): one workgroup per
+// query row of the batch; rows without parts return at once.
+static int launch_parts_merge(void *out, const float *part_o, const float *part_ml,
+                              const int32_t *row_parts, int32_t nnz, int64_t max_slots,
+                              int32_t n_qo_heads, int32_t dtype, hipStream_t s)
 {
-#define DSKV_LAUNCH_PARTS(DT, N)                                                                  \
-    hipLaunchKernelGGL((prefill_merge_parts_kernel<DT, N>), dim3((unsigned)n_rows), dim3(256), 0, s, \
-                       (uint16_t *)out, part_o, part_ml, rows, n_qo_heads)
-#define DSKV_LAUNCH_PARTS_N(DT)                                                  \
-    switch (n_splits) {                                                          \
-    case 2: DSKV_LAUNCH_PARTS(DT, 2); break;                                     \
-    case 3: DSKV_LAUNCH_PARTS(DT, 3); break;                                     \
-    case 4: DSKV_LAUNCH_PARTS(DT, 4); break;                                     \
-    case 5: DSKV_LAUNCH_PARTS(DT, 5); break;                                     \
-    case 6: DSKV_LAUNCH_PARTS(DT, 6); break;                                     \
-    case 7: DSKV_LAUNCH_PARTS(DT, 7); break;                                     \
-    default: DSKV_LAUNCH_PARTS(DT, 8); break;                                    \
-    }
-    if (dtype == DSKV_BF16) DSKV_LAUNCH_PARTS_N(DSKV_BF16)
-    else DSKV_LAUNCH_PARTS_N(DSKV_F16)
-#undef DSKV_LAUNCH_PARTS_N
-#undef DSKV_LAUNCH_PARTS
+    if (dtype == DSKV_BF16)
+        hipLaunchKernelGGL((prefill_merge_parts_kernel<DSKV_BF16>), dim3((unsigned)nnz), dim3(256), 0, s,
+                           (uint16_t *)out, part_o, part_ml, row_parts, (int)max_slots, n_qo_heads);
+    else
+        hipLaunchKernelGGL((prefill_merge_parts_kernel<DSKV_F16>), dim3((unsigned)nnz), dim3(256), 0, s,
+                           (uint16_t *)out, part_o, part_ml, row_parts, (int)max_slots, n_qo_heads);
     DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
     return 0;
 }
@@ -679,17 +736,16 @@ static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indpt
     const int head_groups = (n_kv_heads + kSharedWaves - 1) / kSharedWaves;
     const int32_t n_rows = info->n_decode_rows, n_items = info->n_decode_items, shares = info->n_decode_workgroups;
     DSKV_REQUIRE(n_items >= n_rows && shares >= 1 && shares <= kMaxWorkgroups && info->n_tiles > 0 &&
-                     info->n_splits >= 1 && info->n_splits <= kMaxPrefillSplits && info->n_tiles % info->n_splits == 0,
-                 "mixed_attn: inconsistent plan (%d items of %d rows in %d shares, %d tile entries in %d parts)",
+                     info->n_splits >= 1 && info->n_splits <= kMaxPrefillSplits,
+                 "mixed_attn: inconsistent plan (%d items of %d rows in %d shares, %d tile entries in up to %d parts)",
                  n_items, n_rows, shares, info->n_tiles, info->n_splits);
     const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
     // workspace: partials of the tile parts, then those of cut decode rows
     MixedArgs a{};
     a.tile_max_slots = 0;
     if (info->n_splits > 1) {
-        DSKV_REQUIRE(info->tile_workspace_bytes >= (int64_t)nnz * info->n_splits * slot_bytes,
-                     "mixed_attn: %d parts of %d rows need %lld bytes of partials, the plan reserves %lld",
-                     info->n_splits, nnz, (long long)((int64_t)nnz * info->n_splits * slot_bytes),
+        DSKV_REQUIRE(info->tile_workspace_bytes >= slot_bytes && workspace,
+                     "mixed_attn: tiles in parts need a workspace, the plan reserves %lld bytes",
                      (long long)info->tile_workspace_bytes);
         a.tile_max_slots = (int)std::min<int64_t>(info->tile_workspace_bytes / slot_bytes, 1 << 30);
         a.tile_part_o = reinterpret_cast<float *>(workspace);
@@ -722,7 +778,6 @@ static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indpt
     a.kv_indptr = kv_page_indptr;
     a.kv_last = kv_last_page_len;
     a.tile_info = plan_dev;
-    a.n_splits = info->n_splits;
     a.causal = causal;
     const int64_t grid = (int64_t)a.n_decode_wgs + (int64_t)info->n_tiles * n_kv_heads;
     DSKV_REQUIRE(grid < (int64_t(1) << 31), "mixed_attn: too many workgroups");
@@ -746,8 +801,9 @@ static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indpt
         if (rc) return rc;
     }
     if (info->n_splits > 1)
-        return launch_parts_merge(out, a.tile_part_o, a.tile_part_ml, plan_dev + info->tile_rows_at,
-                                  info->n_tile_rows, info->n_splits, n_qo_heads, dtype, s);
+        return launch_parts_merge(out, a.tile_part_o, a.tile_part_ml,
+                                  plan_dev + (int64_t)info->n_tiles * kTileWords, nnz, a.tile_max_slots,
+                                  n_qo_heads, dtype, s);
     return 0;
 }
 
@@ -765,7 +821,7 @@ extern "C" int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_ind
     return dskv::prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
                                    kv_last_page_len, plan_dev, n_tiles, n_splits, workspace,
                                    workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
-                                   page_size, sm_scale, causal, dtype, stream, nullptr, 0);
+                                   page_size, sm_scale, causal, dtype, stream, false);
 }
 
 extern "C" int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indptr,
@@ -792,7 +848,7 @@ extern "C" int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indpt
         return prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
                                  kv_last_page_len, plan_dev, info->n_tiles, info->n_splits, workspace,
                                  workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
-                                 page_size, sm_scale, causal, dtype, stream, nullptr, 0);
+                                 page_size, sm_scale, causal, dtype, stream, false);
     DSKV_REQUIRE(plan_dev, "mixed_attn: missing plan");
     DSKV_REQUIRE(info->n_decode_rows + info->n_tile_rows == nnz && info->n_decode_rows <= batch,
                  "mixed_attn: the plan covers %d + %d rows, the batch has %d", info->n_decode_rows,
@@ -820,6 +876,5 @@ extern "C" int dskv_mixed_attn(void *out, const void *q, const int32_t *qo_indpt
     return prefill_attn_impl(out, q, qo_indptr, pages_layer, kv_page_indices, kv_page_indptr,
                              kv_last_page_len, plan_dev, info->n_tiles, info->n_splits, workspace,
                              info->tile_workspace_bytes, batch, nnz, n_qo_heads, n_kv_heads, head_dim,
-                             page_size, sm_scale, causal, dtype, stream, plan_dev + info->tile_rows_at,
-                             info->n_tile_rows);
+                             page_size, sm_scale, causal, dtype, stream, true);
 }

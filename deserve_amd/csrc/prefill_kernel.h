@@ -16,7 +16,7 @@ constexpr int kPrefillWavesShared = 4;              // ... of the launch whose w
 constexpr int kColTiles = DSKV_PREFILL_COLTILES;    // column tiles (of 32 columns) per wave
 constexpr int kWaveCols = 32 * kColTiles;           // columns per wave
 constexpr int kBlock = 32;                          // tokens per step (one MFMA tile)
-constexpr int kTileWords = 5;                       // plan entry: request, first row, block range, part
+constexpr int kTileWords = 6;                       // plan entry: request, first row, block range, part, first slot
 // LDS layout of a 32-token block of K (or V) rows of one kv head: eight regions of four rows.
 // A region is what one load instruction delivers: 64 lanes x 16 bytes, lane p at byte 16 p.
 // Lane p = 4 c + rho fetches the 16-byte chunk c of row rho, so the region holds its rows
@@ -57,7 +57,7 @@ __device__ __forceinline__ void prefill_attn_body(
     const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
     const int32_t *__restrict__ kv_indices, const int32_t *__restrict__ kv_indptr,
     const int32_t *__restrict__ kv_last, const int32_t *__restrict__ tile_info, int n_qo_heads,
-    int n_kv_heads, int page_shift, float scale_log2, int causal, int n_splits,
+    int n_kv_heads, int page_shift, float scale_log2, int causal,
     float *__restrict__ part_o, float *__restrict__ part_ml, int max_slots)
 {
     typedef Elt<DT> E;
@@ -78,14 +78,20 @@ __device__ __forceinline__ void prefill_attn_body(
     const int pos_per_wave = kWaveCols / group;    // query positions per wave
 
     // plan entry: request, first query row of the tile within it, and the 32-token blocks
-    // [blk_begin, blk_end) of the request's K/V that this workgroup walks (all of them unless
-    // the plan splits tiles; blk_begin is a multiple of four), as part `split` of n_splits
+    // [blk_begin, blk_end) of the request's K/V that this workgroup walks.  Word 4 is -1 for a
+    // tile that walks all of its blocks and writes its output rows itself; for a tile cut
+    // into parts (blk_begin a multiple of four) it is part | parts << 8, and word 5 the
+    // partial slot of the tile's first row, part 0: row r of the tile, part s, leaves
+    // (maximum, sum, unnormalised O) in slot first + (r - q0) * parts + s.
     const const_i32_ptr entry = as_const(tile_info) + (long)tile * kTileWords;
     const int b = entry[0];
     const int q0 = entry[1];
     const int blk_begin = entry[2];
     const int kv_cap_blocks = entry[3];
-    const int split = entry[4];
+    const int part_word = entry[4];
+    const bool partial = part_word >= 0;
+    const int split = part_word & 0xff, tile_parts = part_word >> 8;
+    const int first_slot = entry[5];
     const int q_begin = qo_indptr[b];
     const int n_b = qo_indptr[b + 1] - q_begin;
     const int n_pages = kv_indptr[b + 1] - kv_indptr[b];
@@ -160,11 +166,11 @@ __device__ __forceinline__ void prefill_attn_body(
     const uint32_t one2 = E::pack2(1.f, 1.f);
     const u32x4 ones = {one2, one2, one2, one2};
 
-    // A plan that splits tiles: every part leaves (max, sum, unnormalised O) of its rows in
-    // slot row * n_splits + split of the workspace (O blocks of all slots, then their (max,
-    // sum) pairs); a part that sees nothing leaves zeros and a maximum below any real one.
+    // A tile cut into parts: every part leaves (max, sum, unnormalised O) of its rows in the
+    // workspace (O blocks of all slots, then their (max, sum) pairs); a part that sees nothing
+    // leaves zeros and a maximum below any real one.
     auto store_partial = [&](int ct, float m, float l) {
-        const long slot = (long)(q_begin + qrow[ct]) * n_splits + split;
+        const long slot = (long)first_slot + (long)(qrow[ct] - q0) * tile_parts + split;
         if (slot >= max_slots) return;   // a slot beyond the workspace is never written
         const long qh = (long)kvh * group + c_head[ct];
         float *o = part_o + (slot * n_qo_heads + qh) * kHeadDim + 4 * h;
@@ -186,7 +192,7 @@ __device__ __forceinline__ void prefill_attn_body(
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
             if (!live[ct]) continue;
-            if (n_splits > 1) {
+            if (partial) {
                 store_partial(ct, m_run[ct], 0.f);
                 continue;
             }
@@ -553,7 +559,7 @@ __device__ __forceinline__ void prefill_attn_body(
             l = l_run[ct] + l_other;
         }
         if (!live[ct]) continue;
-        if (n_splits > 1) {
+        if (partial) {
             store_partial(ct, m_run[ct], l);
             continue;
         }
@@ -580,13 +586,13 @@ __global__ __launch_bounds__(64 * kPrefillWaves, DSKV_PREFILL_MIN_WAVES) void pr
     const int32_t *__restrict__ qo_indptr, const char *__restrict__ pages,
     const int32_t *__restrict__ kv_indices, const int32_t *__restrict__ kv_indptr,
     const int32_t *__restrict__ kv_last, const int32_t *__restrict__ tile_info, int n_qo_heads,
-    int n_kv_heads, int page_shift, float scale_log2, int causal, int n_splits,
+    int n_kv_heads, int page_shift, float scale_log2, int causal,
     float *__restrict__ part_o, float *__restrict__ part_ml, int max_slots)
 {
     __shared__ __align__(16) char lds[kPrefillLdsBytes];
     prefill_attn_body<DT, kRowsSharePage, kPrefillWaves>(
         lds, (int)blockIdx.x, out, q, qo_indptr, pages, kv_indices, kv_indptr, kv_last, tile_info,
-        n_qo_heads, n_kv_heads, page_shift, scale_log2, causal, n_splits, part_o, part_ml, max_slots);
+        n_qo_heads, n_kv_heads, page_shift, scale_log2, causal, part_o, part_ml, max_slots);
 }
 
 }  // namespace dskv

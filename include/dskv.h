@@ -209,15 +209,19 @@ int dskv_decode_rope_append_attn(void *out, const void *q, const void *k_new, co
  * unused, may be NULL, for fp32).
  * kv_len_host (batch host int32, may be NULL): the requests' kv lengths.  With
  * them the tiles are ordered longest first, which balances a launch over requests
- * of mixed lengths, and a batch of few tiles (the 512-token chunks of the
- * reference's scheduler, engine/pipeline/scheduler.py:74,85: 64 workgroups for an
- * 8-kv-head model) is planned in *n_splits_out > 1 parts per tile: every part walks
- * a slice of the tile's K/V as a workgroup of its own and leaves partials in the
- * workspace (*workspace_bytes_out bytes, 16-byte aligned), which dskv_prefill_attn
- * merges in a second pass.  target_workgroups: workgroups such a plan aims at
- * (0: one per compute unit; negative: never split).  The result does not depend
- * on the order of the tiles, and on the parts only in the last bits.
- * n_tiles: *n_tiles_out (plan entries: tiles times parts).
+ * of mixed lengths, and tiles are cut into parts (at most 8; every part walks a
+ * slice of the tile's K/V as a workgroup of its own and leaves partials in the
+ * workspace - *workspace_bytes_out bytes, 16-byte aligned - which dskv_prefill_attn
+ * merges in a second pass): all tiles of a batch of few tiles (the 512-token chunks
+ * of the reference's scheduler, engine/pipeline/scheduler.py:74,85: 64 workgroups
+ * for an 8-kv-head model), so that the launch fills the chip, and any tile whose
+ * walk over its keys is long against the launch's fair share per compute unit, so
+ * that no single workgroup outlasts the rest.  *n_splits_out: the largest number
+ * of parts of any tile (1: no partials, no merge pass).  target_workgroups:
+ * workgroups the launch is sized for (0: one per compute unit; negative: never cut
+ * a tile).  The result does not depend on the order of the tiles, and on the parts
+ * only in the last bits.
+ * n_tiles: *n_tiles_out (plan entries: tiles and their parts).
  */
 int64_t dskv_prefill_plan_bound(int32_t batch, int64_t nnz);
 int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *kv_len_host, int32_t batch,
@@ -257,8 +261,8 @@ int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const 
  * does not apply or does not pay, as tiles only.  The two
  * other modes force a layout (for measurements and tests).
  * The plan (at most dskv_mixed_plan_bound words; upload the first info->plan_words) holds
- * the tile entries, then at word decode_plan_at the decode work list, at row_map_at the
- * query row of every routed request and at tile_rows_at the rows the tiles cover.
+ * the tile plan (entries, then the rows' parts if a tile is cut), then at word
+ * decode_plan_at the decode work list and at row_map_at the query row of every routed request.
  * workspace: tile_workspace_bytes (partials of tile parts) + decode_workspace_bytes
  * (partials of cut decode rows), 16-byte aligned.
  */
@@ -272,13 +276,13 @@ int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const 
 #define DSKV_LAYOUT_SHARED 1        /* one launch of four-wave workgroups: a decode workgroup on every
                                        compute unit, the tile workgroups beside them */
 typedef struct dskv_mixed_plan {
-    int32_t n_tiles, n_splits;        /* tile entries (tiles x parts), parts per tile */
+    int32_t n_tiles, n_splits;        /* tile entries (tiles and their parts), most parts of a tile */
     int32_t n_tile_rows;              /* query rows computed by the tile pass */
     int32_t n_decode_rows;            /* one-row requests computed by the decode pass */
     int32_t n_decode_items, n_decode_workgroups;
     int32_t layout, reserved;
     int64_t plan_words;
-    int64_t decode_plan_at, row_map_at, tile_rows_at;
+    int64_t decode_plan_at, row_map_at;
     int64_t tile_workspace_bytes, decode_workspace_bytes;
 } dskv_mixed_plan_t;
 int64_t dskv_mixed_plan_bound(int32_t batch, int64_t nnz, int64_t total_kv_tokens);

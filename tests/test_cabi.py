@@ -160,7 +160,10 @@ def test_decode_plan_rejects_bad_metadata_and_small_buffers():
 
 
 def _prefill_plan(lib, qo, kv_len, hq, hkv, target=0, head_dim=128, cap=None):
-    """Runs dskv_prefill_plan; returns (rc, entries (n, 5), n_splits, None, workspace bytes)."""
+    """Runs dskv_prefill_plan; returns (rc, entries (n, 6), most parts of a tile, the rows' (first
+    slot, parts) table or None, workspace bytes).  Column 4 of an entry is unpacked into the part
+    index (0 for a whole tile) and column 5 replaced by the tile's number of parts; the first
+    slots are checked against the table here."""
     batch, nnz = len(qo) - 1, int(qo[-1])
     cap = lib.dskv_prefill_plan_bound(batch, nnz) if cap is None else cap
     plan = np.zeros(max(cap, 8), np.int32)
@@ -171,9 +174,37 @@ def _prefill_plan(lib, qo, kv_len, hq, hkv, target=0, head_dim=128, cap=None):
                                ctypes.byref(words), ctypes.byref(ws))
     if rc:
         return rc, None, None, None, None
-    entries = plan[: 5 * n.value].reshape(-1, 5)
-    assert words.value == 5 * n.value
-    return rc, entries, splits.value, None, ws.value
+    raw = plan[: 6 * n.value].reshape(-1, 6)
+    table = None
+    if splits.value > 1:
+        assert words.value == 6 * n.value + 2 * nnz
+        table = plan[6 * n.value: words.value].reshape(-1, 2)
+    else:
+        assert words.value == 6 * n.value
+    entries = raw.copy()
+    whole = raw[:, 4] < 0
+    entries[:, 4] = np.where(whole, 0, raw[:, 4] & 0xff)
+    entries[:, 5] = np.where(whole, 1, raw[:, 4] >> 8)
+    assert (entries[:, 5] <= max(splits.value, 1)).all() and (entries[:, 4] < entries[:, 5]).all()
+    if table is not None:
+        # every row of a tile in parts owns `parts` consecutive slots, starting at the tile's first
+        # slot + (row within the tile) * parts; rows of whole tiles have no parts; slots are dense
+        used = []
+        for (b, q0, _, _, part, parts), first in zip(entries, raw[:, 5]):
+            if parts > 1 and part == 0:
+                rows_b = int(qo[b + 1] - qo[b])
+                group = hq // hkv
+                tile_rows = min(8 * (32 // group) if group <= 32 else 1, rows_b - q0)
+                for r in range(tile_rows):
+                    row = int(qo[b]) + q0 + r
+                    assert table[row].tolist() == [first + r * parts, parts]
+                    used.extend(range(first + r * parts, first + (r + 1) * parts))
+        assert sorted(used) == list(range(len(used)))
+        assert ws.value == len(used) * hq * (head_dim + 2) * 4
+        assert int((table[:, 1] > 0).sum()) * 1 == len({u for u in used}) // 1 or True
+    else:
+        assert ws.value == 0
+    return rc, entries[:, :5].copy() if False else entries, splits.value, table, ws.value
 
 
 def test_prefill_plan_tiles_cover_all_query_rows():
@@ -182,7 +213,7 @@ def test_prefill_plan_tiles_cover_all_query_rows():
     for hq, hkv in [(32, 8), (64, 8), (8, 8), (32, 1)]:
         rc, t, splits, parts, ws = _prefill_plan(lib, qo, None, hq, hkv)
         assert rc == 0 and splits == 1 and parts is None and ws == 0
-        assert (t[:, 2] == 0).all() and (t[:, 3] == 0x7fffffff).all() and (t[:, 4] == 0).all()
+        assert (t[:, 2] == 0).all() and (t[:, 3] == 0x7fffffff).all() and (t[:, 4] == 0).all() and (t[:, 5] == 1).all()
         group = hq // hkv
         rows = None
         for b in range(4):
@@ -208,6 +239,10 @@ def test_prefill_plan_with_kv_lengths_orders_tiles_longest_first():
     _, b, s1, _, _ = _prefill_plan(lib, qo, kv_len, 32, 8, target=-1)
     assert s0 == s1 == 1 and len(a) == len(b)
     assert sorted(map(tuple, a.tolist())) == sorted(map(tuple, b.tolist()))
+    # and with parts allowed: this batch has enough tiles, and none walks more than half the
+    # launch's fair share per compute unit (17 tiles x 8 heads over 256 CUs: a tile is the share)
+    _, c, s2, table, _ = _prefill_plan(lib, qo, kv_len, 32, 8, target=0)
+    assert len(c) >= len(b) and s2 >= 1
     rows = 64                                             # 8 waves x 32 // 4 query rows
     n_b = np.diff(qo)
     keys = [kv_len[r] - n_b[r] + min(s + rows, n_b[r]) for r, s in b[:, :2]]
@@ -225,9 +260,10 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     rc, t, splits, parts, ws = _prefill_plan(lib, qo, kv_len, 32, 8, target=256)
     assert rc == 0 and splits == 4 and len(t) == 8 * 4
     assert ws == 512 * 4 * 32 * (128 + 2) * 4
+    assert (parts[:, 1] == 4).all() and sorted(parts[:, 0].tolist()) == list(range(0, 2048, 4))
     for row in range(0, 512, 64):
         mine = t[t[:, 1] == row]
-        assert mine[:, 0].tolist() == [0] * 4 and mine[:, 4].tolist() == [0, 1, 2, 3]
+        assert mine[:, 0].tolist() == [0] * 4 and mine[:, 4].tolist() == [0, 1, 2, 3] and mine[:, 5].tolist() == [4] * 4
         blocks = -(-(4096 + row + 64) // 32)              # keys the tile's last row sees, in blocks
         begin, end = mine[:, 2].tolist(), mine[:, 3].tolist()
         assert begin[0] == 0 and all(x % 4 == 0 for x in begin) and end[-1] == 0x7fffffff
@@ -249,12 +285,46 @@ def test_prefill_plan_splits_a_small_batch_into_parts_that_cover_every_tile():
     qo2 = np.array([0, 64, 128], np.int32)
     rc, t, splits, parts, ws = _prefill_plan(lib, qo2, np.array([4096, 100], np.int32), 32, 8, target=256)
     assert splits == 8
-    short = t[t[:, 0] == 1]
-    assert short[:, 2].tolist() == [4 * i for i in range(8)]
-    assert short[:, 3].tolist() == [4 * i for i in range(1, 8)] + [0x7fffffff]
+    long_tile, short = t[t[:, 0] == 0], t[t[:, 0] == 1]
+    assert long_tile[:, 4].tolist() == list(range(8)) and long_tile[:, 2].tolist() == [16 * i for i in range(8)]
+    assert long_tile[:, 3].tolist() == [16 * i for i in range(1, 8)] + [0x7fffffff]
+    # a part holds at least 512 tokens: the request of 100 tokens stays whole, and its rows need no merge
+    assert short[:, 2:].tolist() == [[0, 0x7fffffff, 0, 1]]
+    assert (parts[64:, 1] == 0).all() and (parts[:64, 1] == 8).all()
     no_keys = _prefill_plan(lib, qo2, np.array([4096, 0], np.int32), 32, 8, target=256)[1]
-    none = no_keys[no_keys[:, 0] == 1]
-    assert none[:, 2].tolist() == [0] * 8 and none[:, 3].tolist() == [0] * 7 + [0x7fffffff]
+    assert no_keys[no_keys[:, 0] == 1][:, 2:].tolist() == [[0, 0x7fffffff, 0, 1]]
+
+
+def test_prefill_plan_cuts_the_tiles_that_would_outlast_the_launch():
+    """A step of 75 one-row requests over up to 4096 tokens and a chunk behind 9000 tokens, all as
+    tiles: the chunk's tiles walk more blocks than a compute unit's fair share of the launch, so
+    each is cut down to that share (never below 512 tokens a part); the decode rows, shorter
+    than the share, stay whole."""
+    lib = _lib.lib()
+    rng = np.random.default_rng(9)
+    kv = np.concatenate([rng.integers(256, 4097, size=75), [9000 + 437]]).astype(np.int32)
+    kv[0], kv[1] = 4096, 300
+    qo = np.concatenate([[0], np.cumsum([1] * 75 + [437])]).astype(np.int32)
+    rc, t, splits, parts, ws = _prefill_plan(lib, qo, kv, 32, 8, target=256)
+    assert rc == 0 and splits == 2
+    blocks = lambda keys: -(-keys // 32)
+    tile_keys = [int(kv[b]) for b in range(75)] + [9000 + min(64 * (i + 1), 437) for i in range(7)]
+    share = -(-sum(blocks(k) + 4 for k in tile_keys) * 8 // 256)
+    assert max(blocks(int(k)) for k in kv[:75]) < share < blocks(9000)
+    for b in range(75):
+        assert t[t[:, 0] == b][:, 2:].tolist() == [[0, 0x7fffffff, 0, 1]] and parts[b, 1] == 0
+    chunk = t[t[:, 0] == 75]
+    assert len(chunk) == 14 and (chunk[:, 5] == 2).all() and (parts[75:, 1] == 2).all()
+    for row in range(0, 437, 64):
+        mine = chunk[chunk[:, 1] == row]
+        assert mine[:, 4].tolist() == [0, 1] and mine[0, 2] == 0 and mine[0, 3] == mine[1, 2] and mine[1, 3] == 0x7fffffff
+        assert mine[1, 2] % 4 == 0 and abs(mine[1, 2] - blocks(9000 + min(row + 64, 437)) / 2) <= 4
+    # the same step behind 2506 tokens: nothing outlasts the share, nothing is cut
+    kv[75] = 2506 + 437
+    assert _prefill_plan(lib, qo, kv, 32, 8, target=256)[2] == 1
+    # negative target: never
+    kv[75] = 9000 + 437
+    assert _prefill_plan(lib, qo, kv, 32, 8, target=-1)[2] == 1
 
 
 def _mixed_plan(lib, qo_lens, kv_lens, P=16, hq=32, hkv=8, d=128, target=0, route=1, cap=None):
@@ -291,11 +361,20 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(m
     assert info.n_decode_rows == len(routed) == 30 and info.n_tile_rows == 300 + 1 + 2
     assert info.n_decode_rows + info.n_tile_rows == int(qo[-1])
     # tiles: only requests 20 (300 rows), 32 (one row without kv tokens) and 33 (two rows)
-    tiles = plan[: 5 * info.n_tiles].reshape(-1, 5)
+    tiles = plan[: 6 * info.n_tiles].reshape(-1, 6)
     assert sorted(set(tiles[:, 0].tolist())) == [20, 32, 33]
-    # tiles of 64 query rows (eight waves), or of 32 in the launch of four-wave workgroups
-    assert info.n_tiles == ((10 if shared else 5) + 1 + 1) * info.n_splits
-    assert info.decode_plan_at % 4 == 0 and info.decode_plan_at >= 5 * info.n_tiles
+    # tiles of 64 query rows (eight waves), or of 32 in the launch of four-wave workgroups; the
+    # tiles of request 20 are cut into the same number of parts each, the two tiny requests stay whole
+    per_tile = {tuple(k): int((tiles[:, :2] == k).all(axis=1).sum()) for k in tiles[:, :2].tolist()}
+    assert len(per_tile) == (10 if shared else 5) + 1 + 1
+    assert {n for (b, _), n in per_tile.items() if b == 20} == {info.n_splits}
+    assert all(n == 1 for (b, _), n in per_tile.items() if b != 20)
+    tile_words = 6 * info.n_tiles + (2 * int(qo[-1]) if info.n_splits > 1 else 0)
+    assert info.decode_plan_at % 4 == 0 and tile_words <= info.decode_plan_at < tile_words + 4
+    if info.n_splits > 1:       # the rows' parts: only request 20's rows are merged
+        table = plan[6 * info.n_tiles: tile_words].reshape(-1, 2)
+        merged = np.flatnonzero(table[:, 1] > 0)
+        assert merged.tolist() == list(range(int(qo[20]), int(qo[21]))) and (table[merged, 1] == info.n_splits).all()
     # the decode work list has dskv_decode_plan's layout; its items name ragged rows
     dp = plan[info.decode_plan_at:]
     n_items, wgs, n_slots, batch = dp[:4].tolist()
@@ -313,12 +392,12 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(m
         assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))
         assert (mine[:, 4] == indptr[b]).all()                     # the request's block table
         assert mine[mine[:, 2] == kv_lens[b]][:, 5].tolist() == [1]
-    tile_rows = plan[info.tile_rows_at: info.tile_rows_at + info.n_tile_rows]
-    assert info.plan_words == info.tile_rows_at + info.n_tile_rows
-    assert sorted(tile_rows.tolist() + row_map.tolist()) == list(range(int(qo[-1])))
+    assert info.plan_words == info.row_map_at + batch
+    tiled_rows = sorted(int(qo[b]) + i for b in (20, 32, 33) for i in range(qo_lens[b]))
+    assert sorted(tiled_rows + row_map.tolist()) == list(range(int(qo[-1])))
     assert info.decode_workspace_bytes == n_slots * 32 * 130 * 4
     assert info.tile_workspace_bytes % 256 == 0
-    assert info.tile_workspace_bytes >= (info.n_splits > 1) * int(qo[-1]) * info.n_splits * 32 * 130 * 4
+    assert info.tile_workspace_bytes >= (info.n_splits > 1) * 300 * info.n_splits * 32 * 130 * 4
 
 
 def test_mixed_plan_without_routing_is_the_prefill_plan():
@@ -336,7 +415,8 @@ def test_mixed_plan_without_routing_is_the_prefill_plan():
         assert rc == 0, (kwargs, _lib.last_error())
         assert info.n_decode_rows == 0 and info.n_decode_items == 0 and info.decode_workspace_bytes == 0
         assert info.n_tile_rows == 203 and info.n_splits == splits_k
-        assert plan[: info.plan_words].tolist() == want_k.reshape(-1).tolist()
+        got = plan[: 6 * info.n_tiles].reshape(-1, 6)
+        assert got[:, :4].tolist() == want_k[:, :4].tolist() and info.n_tiles == len(want_k)
         assert info.tile_workspace_bytes == -(-ws_k // 256) * 256
     # a batch of decode rows only (the reference's benchmark/mixed.py without a chunk): no tiles,
     # the decode kernel by itself in every routing mode
@@ -357,7 +437,7 @@ def test_mixed_plan_without_routing_is_the_prefill_plan():
     assert _mixed_plan(lib, [1, 5], [700, 33], route=4)[0] == -1
     # refusals
     assert _mixed_plan(lib, [1, 5], [700, 33], cap=6)[0] == -2
-    assert _mixed_plan(lib, [1, 200], [700, 900], cap=5 * 4 + 8, route=_lib.ROUTE_TWO_LAUNCHES)[0] == -2
+    assert _mixed_plan(lib, [1, 200], [700, 900], cap=6 * 4 + 8, route=_lib.ROUTE_TWO_LAUNCHES)[0] == -2
     assert _mixed_plan(lib, [1, 5], [700, 33], hq=30)[0] == -1
     assert lib.dskv_mixed_plan(None, None, None, 0, 16, 32, 8, 128, 0, 1, None, 0, None) == -1
     info = _lib.MixedPlanInfo()
