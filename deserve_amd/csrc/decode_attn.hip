@@ -148,6 +148,148 @@ __global__ __launch_bounds__(64) void decode_attn_generic_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Generic path that shares K/V across the GQA group: fp32 or 16-bit storage, head_dim a
+// multiple of 8 up to 128, groups of up to 8 q heads.  One wavefront per (item, kv head)
+// serves all q heads of the group, so each K/V byte crosses the memory path once (the kernel
+// above reads it once per q head).  Lane (g = lane / 16, c = lane % 16) holds dims 8c .. 8c+7
+// of tokens t + g, t + 4 + g, ...: a token's row is 16 lanes x 32 (or 16) bytes, contiguous;
+// the scores are reduced over the 16 lanes of a row with DPP adds, 16 tokens are in flight per
+// iteration, and the per-group partial sums of O are folded across g once, at the end.
+// The block table entries of an iteration are fetched an iteration ahead.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float row16_sum(float v)
+{
+    // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return v;
+}
+
+template <int DT>
+__device__ __forceinline__ void load_row8(const char *row, bool live, float (&f)[8])
+{
+    // 8 consecutive elements of a K or V row (zeros for a lane beyond head_dim)
+    constexpr int kChunks = 8 / Chunk<DT>::kElems;   // fp32: two 16-byte loads, 16-bit: one
+#pragma unroll
+    for (int i = 0; i < kChunks; i++) {
+        u32x4 raw = {0, 0, 0, 0};
+        if (live) raw = *reinterpret_cast<const u32x4 *>(row + 16 * i);
+        Chunk<DT>::unpack(raw, f + Chunk<DT>::kElems * i);
+    }
+}
+
+template <int DT, int kG>   // kG: q heads per kv head the wave carries (group padded to 1, 2, 4, 8)
+__global__ __launch_bounds__(64) void decode_attn_gqa_kernel(
+    void *__restrict__ out, const void *__restrict__ q, const void *__restrict__ pages,
+    const int32_t *__restrict__ kv_indices, const Item *__restrict__ items,
+    float *__restrict__ part_o, float *__restrict__ part_ml, int max_slots, int n_qo_heads,
+    int n_kv_heads, int head_dim, int page_size, float scale_log2)
+{
+    typedef LoadElt<DT> L;
+    constexpr int kElt = DT == DSKV_F32 ? 4 : 2;
+    constexpr int kSub = 4;                     // sub-steps of 4 tokens per iteration: 16 tokens in flight
+    const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+    const int kvh = blockIdx.y;
+    const int group = n_qo_heads / n_kv_heads;
+    const Item item = items[blockIdx.x];
+    const int b = item.b;
+    const bool live = c * 8 < head_dim;
+    const long row_bytes = (long)n_kv_heads * head_dim * kElt;
+    const long half_bytes = row_bytes * page_size;
+    const long lane_off = ((long)kvh * head_dim + c * 8) * kElt;
+    const char *pool = reinterpret_cast<const char *>(pages);
+    const int32_t *table = kv_indices + item.page_begin;
+
+    float qv[kG][8], acc[kG][8], m_run[kG], l_part[kG];
+#pragma unroll
+    for (int h = 0; h < kG; h++) {
+        m_run[h] = kNegBig;
+        l_part[h] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            acc[h][i] = 0.f;
+            qv[h][i] = (h < group && live)
+                           ? L::get(q, ((long)b * n_qo_heads + (long)kvh * group + h) * head_dim + c * 8 + i) * scale_log2
+                           : 0.f;
+        }
+    }
+    const int last_tok = item.tok_end - 1;
+    // page ids of the lane's tokens of one iteration (past the end: the last token again)
+    auto lookup = [&](int t0, long (&page)[kSub]) {
+#pragma unroll
+        for (int j = 0; j < kSub; j++) page[j] = table[min(t0 + 4 * j + g, last_tok) / page_size];
+    };
+    long page[kSub];
+    if (item.tok_begin < item.tok_end) lookup(item.tok_begin, page);
+    for (int t0 = item.tok_begin; t0 < item.tok_end; t0 += 4 * kSub) {
+        float kx[kSub][8], vx[kSub][8];
+#pragma unroll
+        for (int j = 0; j < kSub; j++) {
+            const int t = min(t0 + 4 * j + g, last_tok);
+            const char *row = pool + page[j] * 2 * half_bytes + (long)(t % page_size) * row_bytes + lane_off;
+            load_row8<DT>(row, live, kx[j]);
+            load_row8<DT>(row + half_bytes, live, vx[j]);
+        }
+        if (t0 + 4 * kSub < item.tok_end) lookup(t0 + 4 * kSub, page);   // for the next turn
+        float x[kG][kSub], m_new[kG];
+#pragma unroll
+        for (int h = 0; h < kG; h++) {
+            float m = m_run[h];
+#pragma unroll
+            for (int j = 0; j < kSub; j++) {
+                float dot = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) dot = __builtin_fmaf(qv[h][i], kx[j][i], dot);
+                x[h][j] = t0 + 4 * j + g <= last_tok ? row16_sum(dot) : kNegBig;
+                m = fmaxf(m, x[h][j]);
+            }
+            m_new[h] = quad_rows_max(m);          // over the four token groups
+        }
+#pragma unroll
+        for (int h = 0; h < kG; h++) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run[h] - m_new[h]);
+            m_run[h] = m_new[h];
+            l_part[h] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[h][i] *= alpha;
+#pragma unroll
+            for (int j = 0; j < kSub; j++) {
+                const float p = x[h][j] > kNegBig ? __builtin_amdgcn_exp2f(x[h][j] - m_new[h]) : 0.f;
+                l_part[h] += p;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[h][i] = __builtin_fmaf(p, vx[j][i], acc[h][i]);
+            }
+        }
+    }
+    // fold the four token groups' partial sums; rows of lanes g == 0 then hold the item's result
+#pragma unroll
+    for (int h = 0; h < kG; h++) {
+        const float l = quad_rows_sum(l_part[h]);
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = quad_rows_sum(acc[h][i]);
+        if (g != 0 || !live || h >= group) continue;
+        const int qh = kvh * group + h;
+        if (item.slot < 0) {
+            const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) L::put(out, ((long)b * n_qo_heads + qh) * head_dim + c * 8 + i, o[i] * inv);
+        } else if (item.slot < max_slots) {
+            float *dst = part_o + ((long)item.slot * n_qo_heads + qh) * head_dim + c * 8;
+#pragma unroll
+            for (int i = 0; i < 8; i++) dst[i] = o[i];
+            if (c == 0) {
+                float *ml = part_ml + ((long)item.slot * n_qo_heads + qh) * 2;
+                ml[0] = m_run[h];
+                ml[1] = l;
+            }
+        }
+    }
+}
+
 // Combine the partials of split requests.  One workgroup of kWaves wavefronts per
 // (request, q head), lane = 2 dims; wave w takes parts w, w + kWaves, ...  Latency-bound,
 // so dependent memory round trips are kept few: (m, l) of up to 64 parts are fetched by
@@ -500,6 +642,28 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
         }
 #undef DSKV_LAUNCH_MFMA
         DSKV_LAUNCH_CHECK("decode_attn_mfma_kernel");
+    } else if (n_qo_heads / n_kv_heads <= 8 && head_dim % 8 == 0 && head_dim <= 128 &&
+               ((uintptr_t)pages_layer % 16 == 0) && ((int64_t)n_kv_heads * head_dim * (dtype == DSKV_F32 ? 4 : 2)) % 16 == 0) {
+        // one wave per (item, kv head) carries the whole GQA group
+        const int group = n_qo_heads / n_kv_heads;
+        dim3 grid((unsigned)n_items, (unsigned)n_kv_heads);
+#define DSKV_LAUNCH_GQA_G(DT, G)                                                                  \
+    hipLaunchKernelGGL((decode_attn_gqa_kernel<DT, G>), grid, dim3(64), 0, s, out, q, pages_layer, \
+                       kv_page_indices, items, part_o, part_ml, (int)max_slots, n_qo_heads,       \
+                       n_kv_heads, head_dim, page_size, scale_log2)
+#define DSKV_LAUNCH_GQA(DT)                                  \
+    do {                                                     \
+        if (group <= 1) DSKV_LAUNCH_GQA_G(DT, 1);            \
+        else if (group <= 2) DSKV_LAUNCH_GQA_G(DT, 2);       \
+        else if (group <= 4) DSKV_LAUNCH_GQA_G(DT, 4);       \
+        else DSKV_LAUNCH_GQA_G(DT, 8);                       \
+    } while (0)
+        if (dtype == DSKV_F32) DSKV_LAUNCH_GQA(DSKV_F32);
+        else if (dtype == DSKV_F16) DSKV_LAUNCH_GQA(DSKV_F16);
+        else DSKV_LAUNCH_GQA(DSKV_BF16);
+#undef DSKV_LAUNCH_GQA
+#undef DSKV_LAUNCH_GQA_G
+        DSKV_LAUNCH_CHECK("decode_attn_gqa_kernel");
     } else {
         dim3 grid((unsigned)n_items, (unsigned)n_qo_heads);
 #define DSKV_LAUNCH_GEN(DT)                                                                       \

@@ -140,6 +140,15 @@ DECODE_CASES = [
     ("f32", [512, 100, 1, 33], 16, 32, 8, 128, "f32", 8),
     ("f32_d64", [200, 17], 8, 8, 2, 64, "f32", 0),
     ("bf16_d64_generic", [200, 17], 16, 8, 2, 64, "bf16", 4),
+    # fp32 / other head dims: one wave per (item, kv head) carries the GQA group (groups up to 8,
+    # head_dim a multiple of 8 up to 128); beyond that one wave per (item, q head)
+    ("f32_d96_group3", [70, 5, 333], 16, 12, 4, 96, "f32", 0),
+    ("f32_mha_d32_page8", [40, 3, 100], 8, 4, 4, 32, "f32", 3),
+    ("f32_group8", [700, 64, 1], 16, 64, 8, 128, "f32", 16),
+    ("f16_d72_group2", [90, 17], 4, 4, 2, 72, "f16", 0),
+    ("f32_group16_per_head", [100, 33], 16, 32, 2, 128, "f32", 0),
+    ("f16_d256_per_head", [50, 7], 16, 4, 2, 256, "f16", 0),
+    ("f32_d100_per_head", [50, 7], 16, 4, 2, 100, "f32", 0),
     ("empty_request", [0, 50], 16, 32, 8, 128, "bf16", 0),
     ("long_single", [33000], 16, 32, 8, 128, "bf16", 0),          # 256 parts: the wide merge
     ("long_and_short", [9000, 50, 1], 16, 32, 8, 128, "f16", 128),
