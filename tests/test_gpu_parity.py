@@ -492,6 +492,10 @@ MIXED_CASES = [
     ("f32_generic_kernel", [100, 37, 64], [1, 20, 1], 16, 32, 8, "f32", 0, 2),
     ("group32_stays_tiled", [100, 37, 64], [1, 20, 1], 16, 32, 1, "bf16", 0, 0),
     ("many_rows", [17 * i % 900 + 1 for i in range(75)] + [4500], [1] * 75 + [437], 16, 32, 8, "bf16", 0, 75),
+    # 16 kv heads: four groups of four per decode share in the shared launch; 2 kv heads: half a wave group
+    ("kv16", [900, 33, 2100, 700], [1, 1, 90, 1], 16, 32, 16, "bf16", 0, 3),
+    ("kv2_group16", [900, 33, 1100, 5], [1, 1, 40, 1], 16, 32, 2, "f16", 0, 3),
+    ("kv1_mqa", [300, 64, 1100], [1, 1, 70], 8, 8, 1, "bf16", 0, 2),
 ]
 
 
