@@ -565,7 +565,7 @@ def mixed_section(seed: int, shapes=("8B", "70B", "8B_chunk_behind_8000"), reps:
         L, Hq = {"8B": (16, 32), "70B": (10, 64), "8B_chunk_behind_8000": (16, 32)}[tag]
         dctx, prior, lens = mixed_step_shape(seed + 60)
         if tag == "8B_chunk_behind_8000":
-            prior = [8000]          # a prompt as long as configuration 4's (the planner then shares the CUs)
+            prior = [8000]          # a prompt as long as configuration 4's
         wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=seed + 61)
         n_dec, nnz = len(dctx), wl.nnz
         tok_bytes = wl.kv_bytes_per_token()

@@ -133,80 +133,6 @@ __global__ __launch_bounds__(64) void prefill_attn_generic_kernel(
     }
 }
 
-// Merge pass of a plan with tiles in parts: output row r, head qh = sum_i w_i O_i / sum_i w_i l_i
-// over the row's partials, w_i = exp2(m_i - max_j m_j).  row_parts[2 r] = the row's first slot,
-// row_parts[2 r + 1] = its number of parts (consecutive slots); 0: the row was written by its
-// tile (or by the decode kernel) and is left alone.  One workgroup per query row; a thread
-// owns 16 consecutive dims of one head and requests all of its parts' values at once.  The
-// decode path's merge kernel, launched with one wave per (row, head), took 11.5 us for the
-// 512 rows of a chunk; this one takes about half.
-template <int DT, int kParts>
-__device__ __forceinline__ void merge_row_parts(uint16_t *__restrict__ out, const float *__restrict__ part_o,
-                                                const float *__restrict__ part_ml, long row, long first,
-                                                int n_qo_heads)
-{
-    typedef Elt<DT> E;
-    for (int idx = threadIdx.x; idx < n_qo_heads * (kHeadDim / 16); idx += blockDim.x) {
-        const int qh = idx / (kHeadDim / 16), d0 = (idx % (kHeadDim / 16)) * 16;
-        f32x4 o[kParts][4];
-        float m[kParts], l[kParts];
-#pragma unroll
-        for (int i = 0; i < kParts; i++) {
-            const long slot = first + i;
-            const float *src = part_o + (slot * n_qo_heads + qh) * kHeadDim + d0;
-#pragma unroll
-            for (int j = 0; j < 4; j++) o[i][j] = *reinterpret_cast<const f32x4 *>(src + 4 * j);
-            const float *ml = part_ml + (slot * n_qo_heads + qh) * 2;
-            m[i] = ml[0];
-            l[i] = ml[1];
-        }
-        float m_all = m[0];
-#pragma unroll
-        for (int i = 1; i < kParts; i++) m_all = fmaxf(m_all, m[i]);
-        f32x4 acc[4] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f},
-                        f32x4{0.f, 0.f, 0.f, 0.f}};
-        float l_all = 0.f;
-#pragma unroll
-        for (int i = 0; i < kParts; i++) {
-            const float w = __builtin_amdgcn_exp2f(m[i] - m_all);
-            l_all += w * l[i];
-#pragma unroll
-            for (int j = 0; j < 4; j++) acc[j] += w * o[i][j];
-        }
-        const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
-        uint16_t *dst = out + (row * n_qo_heads + qh) * kHeadDim + d0;
-#pragma unroll
-        for (int j = 0; j < 4; j += 2) {
-            const u32x4 w4 = {E::pack2(acc[j][0] * inv, acc[j][1] * inv), E::pack2(acc[j][2] * inv, acc[j][3] * inv),
-                              E::pack2(acc[j + 1][0] * inv, acc[j + 1][1] * inv),
-                              E::pack2(acc[j + 1][2] * inv, acc[j + 1][3] * inv)};
-            *reinterpret_cast<u32x4 *>(dst + 4 * j) = w4;
-        }
-    }
-}
-
-template <int DT>
-__global__ __launch_bounds__(256) void prefill_merge_parts_kernel(
-    uint16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
-    const int32_t *__restrict__ row_parts, int max_slots, int n_qo_heads)
-{
-    const long row = blockIdx.x;
-    const const_i32_ptr table = as_const(row_parts) + 2 * row;
-    const int first = table[0], n = table[1];   // uniform over the workgroup
-    if (n <= 0 || first < 0 || first + n > max_slots) return;
-    switch (n) {
-    case 1: merge_row_parts<DT, 1>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 2: merge_row_parts<DT, 2>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 3: merge_row_parts<DT, 3>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 4: merge_row_parts<DT, 4>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 5: merge_row_parts<DT, 5>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 6: merge_row_parts<DT, 6>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 7: merge_row_parts<DT, 7>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    case 8: merge_row_parts<DT, 8>(out, part_o, part_ml, row, first, n_qo_heads); break;
-    default: break;   // the planner never cuts a tile into more parts
-    }
-}
-
 static int prefill_rows_per_tile(int n_qo_heads, int n_kv_heads, int waves)
 {
     const int group = n_qo_heads / n_kv_heads;
@@ -291,11 +217,12 @@ constexpr int kMaxSplitTarget = 1024;        // workgroups a split plan aims at,
 // a workgroup's start and end, in 32-token blocks of walking (for the fair share of a launch)
 constexpr int kTileOverheadBlocks = 4;
 constexpr int32_t kWholeRange = 0x7fffffff;  // blk_end of a tile that is not split
-// kv tokens the one-row requests of a mixed batch must hold together before they get decode
-// workgroups of their own beside the tiles (64 MB of K/V per layer in the 8-kv-head bf16 shape)
-constexpr int64_t kMinSharedLaunchTokens = 16384;
-// ... and kv tokens the longest tiled request must hold (see dskv_mixed_plan)
-constexpr int64_t kMinSharedLaunchTiledKeys = 4096;
+// One-row requests of a mixed batch get decode workgroups of their own beside the tiles when
+// there are at least this many of them ...
+constexpr int kMinSharedLaunchRows = 12;
+// ... and when, run as tiles (one live row per tile), they would be most of the launch's work:
+// a tile is priced at its 32-token blocks plus this much for its start and end.
+constexpr int kTileFixedCostBlocks = 16;
 
 static int compute_units()
 {
@@ -475,9 +402,10 @@ extern "C" int dskv_prefill_plan(const int32_t *qo_indptr_host, const int32_t *k
 extern "C" int64_t dskv_mixed_plan_bound(int32_t batch, int64_t nnz, int64_t total_kv_tokens)
 {
     if (batch < 0 || nnz < 0 || total_kv_tokens < 0) return 0;
-    // tile entries, padding, the decode plan, the row map and the list of tiled rows
+    // tile entries, padding, the decode plan, the row map, the list of tiled rows and the
+    // table of parts per row of a shared launch
     return dskv_prefill_plan_bound(batch, nnz) + 4 + dskv_decode_plan_bound(batch, total_kv_tokens) +
-           (int64_t)batch + nnz + 8;
+           (int64_t)batch + 3 * nnz + 8;
 }
 
 extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_page_indptr_host,
@@ -530,22 +458,33 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     // How the routed rows run.  Without tiled rows: the decode kernel by itself (workgroups of
     // eight waves; 117 us where the same rows take 138 us as tiles).  With both kinds: one
     // launch of four-wave workgroups that share the CUs (pages of at least four tokens: the
-    // tile side then loads straight into LDS) - if the decode rows are worth it (a handful of
-    // short decode rows beside a large batch of chunks stay tiles of the usual launch) and if
-    // a chunk follows a long context: as tiles of one launch, a chunk's 64 rows walk all
-    // their keys in ONE workgroup, and behind 8000 tokens that walk outlasts everything else
-    // (228 us against 175 us shared); behind 2500 tokens the two forms take the same time
-    // (144 and 141 + 10 us of merges), and the plain tiles are kept.
-    int64_t routed_tokens = 0, longest_tiled = 0;
-    for (const DecodeRow &r : rows) routed_tokens += r.len;
-    for (int b = 0; b < batch; b++)
-        if (!routed[b] && qo_indptr_host[b + 1] > qo_indptr_host[b]) longest_tiled = std::max<int64_t>(longest_tiled, kv_len[b]);
+    // tile side then loads straight into LDS) and one merge pass for both - if the decode rows
+    // are worth it.  As a tile, a decode row is a workgroup with one live row of 64 that walks
+    // all of the row's keys by itself; measured over steps of 8 to 75 decode rows beside one to
+    // sixteen chunks (bf16, 8 kv heads, groups of 4 and 8), the shared launch wins by 3-40 %
+    // where these one-row tiles would be at least half of the launch's tile work (blocks walked
+    // plus a fixed cost per tile) and there are a dozen rows or more (75 rows + a 437-token
+    // chunk behind 2506 tokens: 147 against 152 us, behind 8000: 171 against 188; 24 rows behind
+    // 4096: 86 against 126; 75 rows of at most 300 tokens: 53 against 87), and loses 5-10 %
+    // beside a large prefill batch (16 chunks of 512: its four-wave tiles move every K/V row
+    // through the CU twice) or with a handful of rows.
+    const int rows_per_tile = prefill_rows_per_tile(n_qo_heads, n_kv_heads, kPrefillWaves);
+    int64_t decode_cost = 0, tile_cost = 0;
+    for (const DecodeRow &r : rows) decode_cost += (r.len + kBlock - 1) / kBlock + kTileFixedCostBlocks;
+    for (int b = 0; b < batch; b++) {
+        const int64_t n_b = (int64_t)qo_indptr_host[b + 1] - qo_indptr_host[b];
+        if (routed[b] || n_b == 0) continue;
+        for (int64_t r0 = 0; r0 < n_b; r0 += rows_per_tile) {
+            const int64_t keys = std::max<int64_t>(kv_len[b] - n_b + std::min<int64_t>(r0 + rows_per_tile, n_b), 0);
+            tile_cost += (keys + kBlock - 1) / kBlock + kTileFixedCostBlocks;
+        }
+    }
     int layout = DSKV_LAYOUT_SEPARATE;
     if (!rows.empty() && n_tile_rows > 0) {
         const bool can_share = page_size >= 4;
         if (route_one_row_requests == DSKV_ROUTE_SHARED_LAUNCH ||
-            (route_one_row_requests == DSKV_ROUTE_AUTO && routed_tokens >= kMinSharedLaunchTokens &&
-             longest_tiled >= kMinSharedLaunchTiledKeys))
+            (route_one_row_requests == DSKV_ROUTE_AUTO && (int64_t)rows.size() >= kMinSharedLaunchRows &&
+             decode_cost >= tile_cost))
             layout = can_share ? DSKV_LAYOUT_SHARED : DSKV_LAYOUT_SEPARATE;
         if (layout != DSKV_LAYOUT_SHARED && route_one_row_requests != DSKV_ROUTE_TWO_LAUNCHES) {
             // not worth it, or not possible: everything as tiles
@@ -583,8 +522,12 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
                           &info->n_decode_workgroups, &decode_words, &info->decode_workspace_bytes);
     if (rc) return rc;
     info->n_decode_rows = (int32_t)rows.size();
+    const int32_t *req_parts = plan_host + at + kPlanHeaderWords + info->n_decode_workgroups + 1;
     at += decode_words;
-    const int64_t total = at + (int64_t)rows.size();
+    // a shared launch merges the parts of both kinds of rows in one pass: behind the row map, a
+    // table of (first slot, parts) for every row of the batch, the tile parts' slots first
+    const int64_t nnz = qo_indptr_host[batch];
+    const int64_t total = at + (int64_t)rows.size() + (layout == DSKV_LAYOUT_SHARED ? 2 * nnz : 0);
     if (total > capacity_words) {
         set_error("mixed_plan: plan needs %lld words, buffer has %lld", (long long)total,
                   (long long)capacity_words);
@@ -592,6 +535,18 @@ extern "C" int dskv_mixed_plan(const int32_t *qo_indptr_host, const int32_t *kv_
     }
     info->row_map_at = at;
     for (const DecodeRow &r : rows) plan_host[at++] = r.row;
+    if (layout == DSKV_LAYOUT_SHARED) {
+        int32_t *table = plan_host + at;
+        if (info->n_splits > 1) std::copy_n(plan_host + (int64_t)info->n_tiles * kTileWords, 2 * nnz, table);
+        else std::fill_n(table, 2 * nnz, 0);
+        const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
+        const int64_t tile_slots = info->tile_workspace_bytes / slot_bytes;
+        for (size_t i = 0; i < rows.size(); i++) {
+            const int32_t first = req_parts[2 * i], n = req_parts[2 * i + 1];
+            table[2 * (int64_t)rows[i].row] = n > 0 ? (int32_t)(tile_slots + first) : 0;
+            table[2 * (int64_t)rows[i].row + 1] = n > 0 ? n : 0;
+        }
+    }
     info->plan_words = total;
     return 0;
 }
@@ -696,20 +651,15 @@ static int prefill_attn_impl(void *out, const void *q, const int32_t *qo_indptr,
     return 0;
 }
 
-// Merge pass of a tile plan with parts (see prefill_merge_parts_kernel): one workgroup per
-// query row of the batch; rows without parts return at once.
+// Merge pass of a tile plan with parts: one workgroup per query row of the batch (the decode
+// path's merge kernel for rows in a few parts, see merge_kernel.h; one wave per (row, head)
+// took 11.5 us for the 512 rows of a chunk, this about half); rows without parts return at once.
 static int launch_parts_merge(void *out, const float *part_o, const float *part_ml,
                               const int32_t *row_parts, int32_t nnz, int64_t max_slots,
                               int32_t n_qo_heads, int32_t dtype, hipStream_t s)
 {
-    if (dtype == DSKV_BF16)
-        hipLaunchKernelGGL((prefill_merge_parts_kernel<DSKV_BF16>), dim3((unsigned)nnz), dim3(256), 0, s,
-                           (uint16_t *)out, part_o, part_ml, row_parts, (int)max_slots, n_qo_heads);
-    else
-        hipLaunchKernelGGL((prefill_merge_parts_kernel<DSKV_F16>), dim3((unsigned)nnz), dim3(256), 0, s,
-                           (uint16_t *)out, part_o, part_ml, row_parts, (int)max_slots, n_qo_heads);
-    DSKV_LAUNCH_CHECK("prefill_merge_parts_kernel");
-    return 0;
+    return launch_partials_merge(out, part_o, part_ml, row_parts, nullptr, (int)max_slots, nnz, n_qo_heads,
+                                 kHeadDim, dtype, false, s);
 }
 
 // One launch for a batch of decode rows and chunks (layout DSKV_LAYOUT_SHARED), then the two
@@ -740,25 +690,27 @@ static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indpt
                  "mixed_attn: inconsistent plan (%d items of %d rows in %d shares, %d tile entries in up to %d parts)",
                  n_items, n_rows, shares, info->n_tiles, info->n_splits);
     const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
-    // workspace: partials of the tile parts, then those of cut decode rows
+    // workspace: the O partials of the tile parts' slots, then those of the cut decode rows'
+    // slots, then the (maximum, sum) pairs in the same order - one numbering of slots, so that
+    // one merge pass takes both kinds of rows
     MixedArgs a{};
-    a.tile_max_slots = 0;
-    if (info->n_splits > 1) {
-        DSKV_REQUIRE(info->tile_workspace_bytes >= slot_bytes && workspace,
-                     "mixed_attn: tiles in parts need a workspace, the plan reserves %lld bytes",
-                     (long long)info->tile_workspace_bytes);
-        a.tile_max_slots = (int)std::min<int64_t>(info->tile_workspace_bytes / slot_bytes, 1 << 30);
-        a.tile_part_o = reinterpret_cast<float *>(workspace);
-        a.tile_part_ml = a.tile_part_o + (int64_t)a.tile_max_slots * n_qo_heads * head_dim;
-    }
-    char *dec_ws = workspace ? (char *)workspace + info->tile_workspace_bytes : nullptr;
-    const int64_t dec_bytes = workspace ? workspace_bytes - info->tile_workspace_bytes : 0;
-    const int64_t dec_slots = std::min<int64_t>(dec_ws ? dec_bytes / slot_bytes : 0, 1 << 30);
-    DSKV_REQUIRE(n_items == n_rows || dec_slots >= (int64_t)n_items - n_rows + 1,
-                 "mixed_attn: workspace too small for %d decode items of %d rows", n_items, n_rows);
+    const int64_t tile_slots = info->tile_workspace_bytes / slot_bytes;
+    const int64_t dec_slots = info->decode_workspace_bytes / slot_bytes;
+    const int64_t all_slots = tile_slots + dec_slots;
+    DSKV_REQUIRE(all_slots < (int64_t(1) << 30) && all_slots * slot_bytes <= workspace_bytes &&
+                     (all_slots == 0 || workspace),
+                 "mixed_attn: the plan's %lld partial slots need %lld bytes of workspace, got %lld",
+                 (long long)all_slots, (long long)(all_slots * slot_bytes), (long long)workspace_bytes);
+    DSKV_REQUIRE(info->n_splits == 1 || tile_slots >= 2, "mixed_attn: tiles in parts without partial slots");
+    DSKV_REQUIRE(n_items == n_rows || dec_slots >= 2, "mixed_attn: cut decode rows without partial slots");
+    float *const part_o = reinterpret_cast<float *>(workspace);
+    float *const part_ml = part_o ? part_o + all_slots * n_qo_heads * (int64_t)head_dim : nullptr;
+    a.tile_max_slots = (int)tile_slots;
+    a.tile_part_o = part_o;
+    a.tile_part_ml = part_ml;
     a.dec_max_slots = (int)dec_slots;
-    a.dec_part_o = reinterpret_cast<float *>(dec_ws);
-    a.dec_part_ml = a.dec_part_o ? a.dec_part_o + dec_slots * n_qo_heads * (int64_t)head_dim : nullptr;
+    a.dec_part_o = part_o ? part_o + tile_slots * n_qo_heads * (int64_t)head_dim : nullptr;
+    a.dec_part_ml = part_ml ? part_ml + tile_slots * n_qo_heads * 2 : nullptr;
     const int32_t *dplan = plan_dev + info->decode_plan_at;
     a.wg_ptr = dplan + kPlanHeaderWords;
     const int32_t *req_parts = a.wg_ptr + shares + 1;
@@ -794,15 +746,21 @@ static int mixed_shared_launch(void *out, const void *q, const int32_t *qo_indpt
     }
 #undef DSKV_LAUNCH_MIXED
     DSKV_LAUNCH_CHECK("mixed_attn_kernel");
-    if (n_items > n_rows) {
-        const bool wide = (int64_t)n_items > 32 * (int64_t)n_rows;
+    // Rows cut into dozens of parts (a few very long decode rows): the decode path's wide merge
+    // for them, then the tile parts' own pass.  Otherwise one pass over the table of all rows.
+    const bool wide = (int64_t)n_items > 32 * (int64_t)n_rows;
+    if (wide) {
         int rc = launch_partials_merge(out, a.dec_part_o, a.dec_part_ml, req_parts, plan_dev + info->row_map_at,
-                                       a.dec_max_slots, n_rows, n_qo_heads, head_dim, dtype, wide, s);
+                                       a.dec_max_slots, n_rows, n_qo_heads, head_dim, dtype, true, s);
         if (rc) return rc;
+        if (info->n_splits > 1)
+            return launch_parts_merge(out, a.tile_part_o, a.tile_part_ml,
+                                      plan_dev + (int64_t)info->n_tiles * kTileWords, nnz, a.tile_max_slots,
+                                      n_qo_heads, dtype, s);
+        return 0;
     }
-    if (info->n_splits > 1)
-        return launch_parts_merge(out, a.tile_part_o, a.tile_part_ml,
-                                  plan_dev + (int64_t)info->n_tiles * kTileWords, nnz, a.tile_max_slots,
+    if (n_items > n_rows || info->n_splits > 1)
+        return launch_parts_merge(out, part_o, part_ml, plan_dev + info->row_map_at + n_rows, nnz, all_slots,
                                   n_qo_heads, dtype, s);
     return 0;
 }

@@ -254,15 +254,18 @@ int dskv_prefill_attn(void *out, const void *q, const int32_t *qo_indptr, const 
  * dskv_prefill_plan / dskv_prefill_attn.  fp32 data is computed by the generic kernel,
  * whatever the plan routed.
  * With DSKV_ROUTE_AUTO a batch of one-row requests only runs the decode pass alone; a batch
- * of both kinds runs as ONE launch (DSKV_LAYOUT_SHARED: pages of at least 4 tokens, one-row
- * requests holding at least 16384 kv tokens together, a tiled request of at least 4096 kv
- * tokens) in which every compute unit hosts a decode workgroup, which keeps its memory path
- * busy, and tile workgroups beside it, which use its matrix pipeline - or, where that launch
- * does not apply or does not pay, as tiles only.  The two
- * other modes force a layout (for measurements and tests).
+ * of both kinds runs as ONE launch (DSKV_LAYOUT_SHARED: pages of at least 4 tokens, at least
+ * 12 one-row requests, which as query tiles of their own would be at least half of the launch's
+ * work) in which every compute unit hosts a decode workgroup, which keeps its memory path
+ * busy, and tile workgroups beside it, which use its matrix pipeline, followed by one merge
+ * pass for both kinds of rows - or, where that launch does not apply or does not pay (a handful
+ * of decode rows, a large prefill batch), as tiles only.  The two other modes force a layout
+ * (for measurements and tests).
  * The plan (at most dskv_mixed_plan_bound words; upload the first info->plan_words) holds
  * the tile plan (entries, then the rows' parts if a tile is cut), then at word
- * decode_plan_at the decode work list and at row_map_at the query row of every routed request.
+ * decode_plan_at the decode work list and at row_map_at the query row of every routed request;
+ * a DSKV_LAYOUT_SHARED plan ends with the parts of every row of the batch (first slot, parts;
+ * the tile parts' slots numbered first), so that ONE merge pass finishes both kinds of rows.
  * workspace: tile_workspace_bytes (partials of tile parts) + decode_workspace_bytes
  * (partials of cut decode rows), 16-byte aligned.
  */

@@ -354,7 +354,7 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(m
     kv_lens = list(rng.integers(200, 4000, size=20)) + [4500] + list(rng.integers(1, 50, size=10)) + [40, 0, 2]
     rc, info, plan, qo, indptr = _mixed_plan(lib, qo_lens, kv_lens, route=mode)
     assert rc == 0, _lib.last_error()
-    # 30 decode rows with more than 16384 kv tokens beside tiles: one shared launch unless told otherwise
+    # 30 decode rows that would outweigh the chunk's five tiles as tiles of their own: one shared launch unless told otherwise
     shared = mode != _lib.ROUTE_TWO_LAUNCHES
     assert info.layout == (_lib.LAYOUT_SHARED if shared else _lib.LAYOUT_SEPARATE)
     routed = [b for b in range(len(qo_lens)) if qo_lens[b] == 1 and kv_lens[b] > 0]
@@ -392,7 +392,27 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(m
         assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))
         assert (mine[:, 4] == indptr[b]).all()                     # the request's block table
         assert mine[mine[:, 2] == kv_lens[b]][:, 5].tolist() == [1]
-    assert info.plan_words == info.row_map_at + batch
+    nnz = int(qo[-1])
+    assert info.plan_words == info.row_map_at + batch + (2 * nnz if shared else 0)
+    if shared:
+        # one merge pass for both kinds of rows: a table of (first slot, parts) per row of the
+        # batch, the tile parts' slots numbered first, the cut decode rows' slots behind them
+        both = plan[info.row_map_at + batch: info.plan_words].reshape(-1, 2)
+        tile_slots = info.tile_workspace_bytes // (32 * 130 * 4)
+        req = dp[4 + wgs + 1: 4 + wgs + 1 + 2 * batch].reshape(-1, 2)
+        for i, b in enumerate(routed):
+            first, n = req[i].tolist()
+            assert both[int(qo[b])].tolist() == ([tile_slots + first, n] if n > 0 else [0, 0])
+        chunk = np.arange(int(qo[20]), int(qo[21]))
+        if info.n_splits > 1:
+            assert (both[chunk, 1] == info.n_splits).all() and both[chunk, 0].max() < tile_slots
+            assert (both[chunk] == table[chunk]).all()
+        else:
+            assert (both[chunk] == 0).all()
+        assert (both[[int(qo[32]), int(qo[33]), int(qo[33]) + 1]] == 0).all()
+        used = both[both[:, 1] > 0]
+        spans = sorted((int(f), int(f + n)) for f, n in used)
+        assert all(x[1] <= y[0] for x, y in zip(spans, spans[1:]))       # no slot belongs to two rows
     tiled_rows = sorted(int(qo[b]) + i for b in (20, 32, 33) for i in range(qo_lens[b]))
     assert sorted(tiled_rows + row_map.tolist()) == list(range(int(qo[-1])))
     assert info.decode_workspace_bytes == n_slots * 32 * 130 * 4

@@ -401,19 +401,20 @@ def test_mixed_step_full_size_through_batch_prefill():
     """The reference's usual step in its decode-first aggregated mode: 75 running requests
     (contexts U[256, 4096], one new token each) and one chunk that fills the 512-token budget
     over a prior of U[0, 4096] tokens, all through BatchPrefill (engine/microbatch/processor.py:
-    116-145) at the Llama-3-8B stage shape (the chunk behind 4200 tokens: one launch in which
-    decode workgroups and query tiles share the compute units) and at the 70B shape (behind
-    1500 tokens: all rows as tiles, the planner's choice there).  EVERY row of the ragged output of
+    116-145) at the Llama-3-8B stage shape (the chunk behind 4200 tokens, its tiles in parts)
+    and at the 70B shape (behind 1500 tokens) - the planner runs both as one launch in which
+    decode workgroups and query tiles share the compute units - and a step of 8 running requests
+    and a 504-token chunk, which it runs as tiles only.  EVERY row of the ragged output of
     two layers against the C oracle, each row against its own scale; the appended rows read
     back bit for bit; the layer's checksum moves by exactly the appended rows."""
     from deserve_amd.execution.exec import BatchPrefill, get_wrappers
     from deserve_amd.synthetic import make_mixed_workload, mixed_step_shape
 
-    for tag, L, Hq in (("8B", 3, 32), ("70B", 2, 64)):
+    for tag, L, Hq in (("8B", 3, 32), ("70B", 2, 64), ("8B_few_rows", 2, 32)):
         _announce("mixed step", tag)
         P, Hkv, D = 16, 8, 128
-        dctx, prior, lens = mixed_step_shape(11)
-        prior[0] = 4200 if tag == "8B" else 1500                        # the planner's two choices: one launch / tiles
+        dctx, prior, lens = mixed_step_shape(11, decode_rows=8 if tag == "8B_few_rows" else 75)
+        prior[0] = 4200 if tag == "8B" else 1500
         wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=11)
         nnz, n_dec = wl.nnz, len(dctx)
         assert nnz == 512
@@ -422,11 +423,11 @@ def test_mixed_step_full_size_through_batch_prefill():
         step.prepare()
         ctx = step.prefill_ctx
         _, w = get_wrappers(DEV)
-        if tag == "8B":     # behind 4200 tokens: one launch, decode rows on the decode kernel, the chunk in parts
-            assert w._info.layout == 1 and w._n_decode_rows == n_dec and w._info.n_tile_rows == nnz - n_dec
-            assert w._n_splits > 1
-        else:               # behind 1500 tokens: every row a tile of the usual launch
+        if tag == "8B_few_rows":     # a handful of decode rows: every row a tile of the usual launch
             assert w._info.layout == 0 and w._n_decode_rows == 0 and w._info.n_tile_rows == nnz
+        else:                        # one launch, decode rows on the decode kernel's body, one merge pass
+            assert w._info.layout == 1 and w._n_decode_rows == n_dec and w._info.n_tile_rows == nnz - n_dec
+            assert w._n_splits > 1 or tag != "8B"
         indptr, ids_all = ctx.host["kv_page_indptr"].numpy(), ctx.host["kv_page_indices"].numpy()
         last, qo = ctx.host["kv_last_page_lens"].numpy(), ctx.host["indptr"].numpy()
         start = np.array([t.start_pos for t in wl.tasks])
