@@ -597,6 +597,7 @@ static int decode_attn_impl(void *out, const void *q, const void *pages_layer,
     // or beyond max_slots, so an undersized workspace can never be overrun.
     const int64_t slot_bytes = (int64_t)n_qo_heads * (head_dim + 2) * (int64_t)sizeof(float);
     DSKV_REQUIRE(workspace_bytes >= 0, "decode_attn: negative workspace size");
+    DSKV_REQUIRE((uintptr_t)workspace % 16 == 0, "decode_attn: the workspace must be 16-byte aligned");
     const int64_t max_slots = std::min<int64_t>(workspace ? workspace_bytes / slot_bytes : 0, 1 << 30);
     DSKV_REQUIRE(n_items == batch || max_slots >= (int64_t)n_items - batch + 1,
                  "decode_attn: workspace (%lld bytes) too small for %d items of %d requests",

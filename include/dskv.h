@@ -99,7 +99,7 @@ int dskv_upload_words(void *dst, const void *src_pinned, int64_t n_words, void *
  *   plan_capacity_words: size of plan_host; dskv_decode_plan_bound(batch,
  *                        total_tokens) words always suffice.
  *   workspace_bytes_out: device scratch dskv_decode_attn needs for the partial
- *                        results of requests that were cut.
+ *                        results of requests that were cut (16-byte aligned).
  */
 int64_t dskv_decode_plan_bound(int32_t batch, int64_t total_tokens);
 int dskv_decode_plan(const int32_t *kv_page_indptr_host, const int32_t *kv_last_page_len_host,

@@ -152,6 +152,9 @@ DECODE_CASES = [
     ("empty_request", [0, 50], 16, 32, 8, 128, "bf16", 0),
     ("long_single", [33000], 16, 32, 8, 128, "bf16", 0),          # 256 parts: the wide merge
     ("long_and_short", [9000, 50, 1], 16, 32, 8, 128, "f16", 128),
+    # more than 8 parts of one request among short ones: the row merge's loop, four parts at a time
+    ("one_long_among_short", [9000, 50, 1, 300, 17, 64, 5, 700], 16, 32, 8, 128, "bf16", 64),
+    ("ten_parts", [2600, 40], 16, 32, 8, 128, "f16", 10),
 ]
 
 
