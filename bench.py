@@ -596,6 +596,8 @@ def mixed_section(seed: int, shapes=("8B", "70B", "8B_chunk_behind_8000"), reps:
         append_us = median_us(lambda l: append_paged_kv_cache(wl.k[l], wl.v[l], c.indptr, wl.pool.pages[l],
                                                               c.kv_page_indices, c.kv_page_indptr,
                                                               c.kv_last_page_lens))
+        # (the first passes over a fresh pool run a few percent slow: one untimed round first)
+        median_us(lambda l: w.forward(wl.q[l], wl.pool.pages[l], causal=True))
         mixed_us = median_us(lambda l: w.forward(wl.q[l], wl.pool.pages[l], causal=True))
         w.end_forward()
         # the whole step as the engine runs it: plan + upload, then L x (append + attention)
