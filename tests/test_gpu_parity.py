@@ -499,6 +499,9 @@ MIXED_CASES = [
     ("kv16", [900, 33, 2100, 700], [1, 1, 90, 1], 16, 32, 16, "bf16", 0, 3),
     ("kv2_group16", [900, 33, 1100, 5], [1, 1, 40, 1], 16, 32, 2, "f16", 0, 3),
     ("kv1_mqa", [300, 64, 1100], [1, 1, 70], 8, 8, 1, "bf16", 0, 2),
+    # a decode row cut into hundreds of parts: the shared launch then merges the decode rows with
+    # eight waves per (row, head) and the tile parts in a pass of their own
+    ("long_row_wide_merge", [33000, 20, 1500], [1, 1, 64], 16, 32, 8, "bf16", 0, 2),
 ]
 
 
@@ -538,6 +541,8 @@ def test_mixed_batch_routes_one_row_requests_to_the_decode_kernel(case):
             assert not shared and w._n_decode_rows == 0
         if name == "cut_rows" and route in (_lib.ROUTE_SHARED_LAUNCH, _lib.ROUTE_TWO_LAUNCHES):
             assert w._info.n_decode_items > w._n_decode_rows          # rows cut across workgroups: merged
+        if name == "long_row_wide_merge" and route in (_lib.ROUTE_SHARED_LAUNCH, _lib.ROUTE_TWO_LAUNCHES):
+            assert w._info.n_decode_items > 32 * w._n_decode_rows     # dozens of parts per row: the wide merge
         for causal in (True, False):
             out = torch.full_like(q, float("nan"))
             assert w.forward(q, pages, causal=causal, out=out) is out
