@@ -53,15 +53,15 @@ struct LoadCursor {
 #ifndef DSKV_DECODE_MIN_WAVES
 #define DSKV_DECODE_MIN_WAVES 1
 #endif
-// kPagesPerTile: pages a 16-token tile spans - 1 (pages of 16 tokens or more: one buffer
-// descriptor per tile), 2 (pages of 8 tokens: the two page ids as scalars, selected per
-// lane), 0 (smaller pages: every lane looks its page up itself; with four scalar ids and a
-// four-way selection pages of 4 tokens were slower than that, 130 against 113 us).
 // The kernel's body for one workgroup: share `share` of the plan, kv heads head_group *
 // kWaves .. + kWaves (one per wave); `lds_base`: kWaves * kVTileBytes of the workgroup's LDS.
 // A function, so that one launch can hold workgroups of this kind next to others.
-// kRing: tiles in flight per wave (one consumed, the rest loading).
-template <int DT, int kPagesPerTile, int kWaves, int kRing = kStages>   // kPagesPerTile: 1, 2 or 0
+//   kPagesPerTile: pages a 16-token tile spans - 1 (pages of 16 tokens or more: one buffer
+//     descriptor per tile), 2 (pages of 8 tokens: the two page ids as scalars, selected per
+//     lane), 0 (smaller pages: every lane looks its page up itself; with four scalar ids and
+//     a four-way selection pages of 4 tokens were slower than that, 130 against 113 us).
+//   kRing: tiles in flight per wave (one consumed, the rest loading).
+template <int DT, int kPagesPerTile, int kWaves, int kRing = kStages>
 __device__ __forceinline__ void decode_attn_body(
     char *lds_base, int share, int head_group, uint16_t *__restrict__ out,
     const uint16_t *__restrict__ q, const char *pages, const int32_t *__restrict__ kv_indices,
