@@ -62,7 +62,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="skip the replayed-graph variant of the step")
     ap.add_argument("--no-mixed", action="store_true", help="skip the mixed decode + chunk section")
     ap.add_argument("--no-page8", action="store_true", help="skip configuration 2 on 8-token pages")
-    ap.add_argument("--section", choices=["swap", "fragmented", "prefill", "mixed", "mfma-ceiling"], default=None,
+    ap.add_argument("--section", choices=["swap", "fragmented", "prefill", "mixed", "mfma-ceiling", "power"],
+                    default=None,
                     help="(internal) run only this host-link section and print its JSON object")
     ap.add_argument("--page-size", type=int, default=16,
                     help="tokens per page of the benched pool (BASELINE's configurations use 16; the "
@@ -540,6 +541,199 @@ def mfma_ceiling_section(seed: int, levels=(0, 1, 2), fills=("normal", "constant
     return out
 
 
+class _BoardSensors:
+    """The board's own sensors through sysfs (the files `amd-smi metric --power --clock` reads):
+    socket power in watts, its cap, and the shader clock in MHz; None where the box exposes no
+    such file.  A sampling thread reads them every 50 ms while a workload runs."""
+
+    def __init__(self):
+        import glob
+        first = lambda pat: (sorted(glob.glob(pat)) or [None])[0]
+        base = "/sys/class/drm/card*/device/hwmon/hwmon*/"
+        self.power = first(base + "power1_input") or first(base + "power1_average")
+        self.cap = first(base + "power1_cap")
+        self.sclk = first(base + "freq1_input")
+        self.dpm_sclk = first("/sys/class/drm/card*/device/pp_dpm_sclk")   # levels, the current one starred
+
+    @staticmethod
+    def _read(path, scale):
+        try:
+            with open(path) as f:
+                return int(f.read().strip()) / scale
+        except (OSError, ValueError, TypeError):
+            return None
+
+    def cap_watts(self):
+        return self._read(self.cap, 1e6)
+
+    def _starred_mhz(self):
+        try:
+            with open(self.dpm_sclk) as f:
+                for line in f:
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().split("mhz")[0])
+        except (OSError, ValueError, TypeError, IndexError):
+            pass
+        return None
+
+    def sample(self):
+        clock = self._read(self.sclk, 1e6)
+        return self._read(self.power, 1e6), clock if clock is not None else self._starred_mhz()
+
+
+def power_section(seed: int, seconds: float = 6.0):
+    """Socket power and shader clock while a kernel runs back to back for `seconds` (sampled
+    from the second 1.5 on, when clock and power have settled): the prefill attention of
+    configuration 4, the bare MFMA loop on N(0,1) and on constant operands, and the decode
+    attention of configuration 2.  Says whether a kernel's rate is what the board's power cap
+    leaves of the nominal clock."""
+    import ctypes
+    import threading
+
+    import numpy as np
+    import torch
+
+    from deserve_amd.execution.exec import get_wrappers
+    from deserve_amd.kvcache.paged.kvcache import PagedKVCache
+    from deserve_amd.kvcache.paged.page_pool import GpuPagePool
+    from deserve_amd.kvcache.paged.page_table import PageTableAllocator
+    from deserve_amd.model.context.flash import FlashDecodeCtx, FlashPrefillCtx
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+    from deserve_amd.synthetic import fill_normal, make_decode_workload, scatter_pool_order
+    from deserve_amd.task import SamplingParams, TaskData
+
+    dev = torch.device("cuda")
+    sensors = _BoardSensors()
+    out = {"sensors": {"power": sensors.power, "cap": sensors.cap, "shader_clock": sensors.sclk or sensors.dpm_sclk},
+           "power_cap_W": sensors.cap_watts(), "seconds_per_workload": seconds,
+           "idle_W": None, "workloads": {}}
+    torch.cuda.synchronize()
+    time.sleep(1.0)
+    out["idle_W"] = sensors.sample()[0]
+
+    def sustained(name, launch, work_per_launch, unit, what):
+        """launch() enqueues some 10-50 ms of the kernel; work_per_launch in flop or bytes."""
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            t0 = time.perf_counter()
+            while not stop.is_set():
+                w_, f_ = sensors.sample()
+                samples.append((time.perf_counter() - t0, w_, f_))
+                time.sleep(0.05)
+
+        th = threading.Thread(target=sampler, daemon=True)
+        th.start()
+        t0 = time.perf_counter()
+        n_settled, t_settled = 0, None
+        while time.perf_counter() - t0 < seconds:
+            launch()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t0 >= 1.5:
+                if t_settled is None:
+                    t_settled = time.perf_counter()
+                else:
+                    n_settled += 1
+        t_end = time.perf_counter()
+        stop.set()
+        th.join()
+        watts = [w_ for t_, w_, _ in samples if t_ >= 1.5 and w_ is not None]
+        clocks = [f_ for t_, _, f_ in samples if t_ >= 1.5 and f_ is not None]
+        rate = work_per_launch * n_settled / (t_end - t_settled) if t_settled and n_settled else None
+        out["workloads"][name] = {
+            "what": what,
+            "rate": round(rate / (1e12 if unit == "TFLOP/s" else 1e9), 1) if rate else None, "unit": unit,
+            "socket_power_W_avg": round(sum(watts) / len(watts), 1) if watts else None,
+            "socket_power_W_max": round(max(watts), 1) if watts else None,
+            "shader_clock_MHz_avg": round(sum(clocks) / len(clocks), 1) if clocks else None,
+            "samples": len(watts)}
+        time.sleep(1.0)           # let the board settle before the next workload
+
+    # prefill attention, configuration 4 (as prefill_section builds it)
+    L, P, Hq, Hkv, D, B, n = 4, 16, 32, 8, 128, 16, 512
+    rng = np.random.default_rng(seed + 40)
+    prior = (rng.integers(0, 8193, size=B) // P) * P + rng.integers(0, 16, size=B)
+    pool = GpuPagePool(L, int((-(-(prior + n) // P)).sum()) + 8, P, dev, torch.bfloat16)
+    fill_normal(pool.pages, seed + 41)
+    scatter_pool_order(pool, seed + 42)
+    rows = PageTableAllocator(B, 8192 + 1024, P, dev)
+    tasks = [TaskData(f"p{b}", int(prior[b]), 1, n, int(prior[b]) + n, SamplingParams()) for b in range(B)]
+    caches = [PagedKVCache.empty(rows, pool) for _ in range(B)]
+    gen = torch.Generator(device="cuda").manual_seed(seed + 43)
+    q = torch.randn((L, B * n, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(1 << 20, dtype=torch.uint8, device=dev))
+    c = FlashPrefillCtx.init_paged_prefill_ctx(tasks, caches, w)
+    w.begin_forward(qo_indptr=c.indptr, paged_kv_indptr=c.kv_page_indptr, paged_kv_indices=c.kv_page_indices,
+                    paged_kv_last_page_len=c.kv_last_page_lens, num_qo_heads=Hq, num_kv_heads=Hkv, head_dim=D,
+                    page_size=P, qo_indptr_host=c.host["indptr"], paged_kv_indptr_host=c.host["kv_page_indptr"],
+                    paged_kv_last_page_len_host=c.host["kv_last_page_lens"],
+                    paged_kv_indices_host=c.host["kv_page_indices"])
+    flops = 4 * Hq * D * sum(n * int(p_) + n * (n + 1) // 2 for p_ in prior)
+    out_rows = torch.empty_like(q[0])
+
+    def prefill_launch():
+        for _ in range(8):
+            for layer in range(L):
+                w.forward(q[layer], pool.pages[layer], causal=True, out=out_rows)
+
+    sustained("prefill_attention_config4", prefill_launch, 32 * flops, "TFLOP/s",
+              "prefill_attn_mfma_kernel<bf16> on configuration 4's 16 x 512-token chunks, N(0,1) q, K, V")
+    q.zero_()
+    pool.pages.zero_()
+    sustained("prefill_attention_config4_zero_data", prefill_launch, 32 * flops, "TFLOP/s",
+              "the same launches over all-zero q, K and V")
+    w.end_forward()
+    del pool, q, w, c, caches, rows
+    torch.cuda.empty_cache()
+
+    # the bare matrix loop
+    path = os.path.join(ROOT, "deserve_amd", "libdskv_calib.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it (python -c 'import __graft_entry__ as g; g.build()')")
+    lib = ctypes.CDLL(path)
+    lib.dskv_calib_mfma_loop.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+    lib.dskv_calib_mfma_loop_flops.restype = ctypes.c_double
+    lib.dskv_calib_mfma_loop_flops.argtypes = [ctypes.c_int, ctypes.c_int]
+    wgs, iters = 1024, 1536
+    g = torch.Generator(device=dev).manual_seed(seed + 70)
+    data = {"normal": torch.randn(512 * 128, generator=g, device=dev).to(torch.bfloat16),
+            "constant": torch.full((512 * 128,), 1.0, device=dev, dtype=torch.bfloat16)}
+    sink = torch.empty(wgs * 512, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    loop_flops = lib.dskv_calib_mfma_loop_flops(wgs, iters)
+    for fill in ("normal", "constant"):
+        def mfma_launch(fill=fill):
+            rc = lib.dskv_calib_mfma_loop(data[fill].data_ptr(), sink.data_ptr(), 0, wgs, iters, 0.1275, stream)
+            if rc != 0:
+                raise RuntimeError(f"dskv_calib_mfma_loop failed with code {rc}")
+        sustained(f"mfma_only_{fill}_operands", mfma_launch, loop_flops, "TFLOP/s",
+                  f"nothing but v_mfma_f32_32x32x16_bf16, {fill} operands, two waves per SIMD")
+
+    # decode attention, configuration 2
+    Ld = 4
+    ctx = np.random.default_rng(seed).integers(256, 4097, size=64)
+    wl = make_decode_workload("power", ctx, Ld, 32, 8, 128, 16, torch.bfloat16, headroom_tokens=32,
+                              seed=seed + 1, fill=True)
+    wd, _ = get_wrappers(wl.pool.main_device)
+    cd = FlashDecodeCtx.init_paged_decode_ctx(wl.tasks, wl.caches, wd)
+    wd.begin_forward(indptr=cd.kv_page_indptr, indices=cd.kv_page_indices, last_page_len=cd.kv_last_page_lens,
+                     num_qo_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
+                     indptr_host=cd.host["kv_page_indptr"], last_page_len_host=cd.host["kv_last_page_lens"])
+    kv_bytes = sum(t.start_pos + 1 for t in wl.tasks) * wl.kv_bytes_per_token()
+    outs = [torch.empty_like(wl.q[0]) for _ in range(Ld)]
+
+    def decode_launch():
+        for _ in range(32):
+            for layer in range(Ld):
+                wd.forward(wl.q[layer], wl.pool.pages[layer], out=outs[layer])
+
+    sustained("decode_attention_config2", decode_launch, 32 * Ld * kv_bytes, "GB/s",
+              "decode_attn_mfma_kernel<bf16> + merge on configuration 2's 64 requests (K/V bytes only)")
+    wd.end_forward()
+    return out
+
+
 def mixed_section(seed: int, shapes=("8B", "70B", "8B_chunk_behind_8000"), reps: int = 6):
     """The reference's usual step in its decode-first aggregated mode (engine/pipeline/stage/
     join.py:11-88, 512-token budget; deserve_exp/exp_args.csv: microbatch size 75): 75 running
@@ -841,6 +1035,8 @@ def main() -> int:
                                              config4=not a.prefill_one_chunk_only)))
         elif a.section == "mfma-ceiling":
             print(json.dumps(mfma_ceiling_section(a.seed)))
+        elif a.section == "power":
+            print(json.dumps(power_section(a.seed)))
         elif a.section == "mixed":
             print(json.dumps(mixed_section(a.seed, shapes=tuple(a.mixed_shapes.split(",")))))
         else:
