@@ -1,9 +1,9 @@
 // Rotary position embedding on the ragged q/k of one step, adjacent-pair
 // ("interleaved") convention: (x[2j], x[2j+1]) is rotated by
 // pos * theta^(-2j/D) with pos = offsets[request] + index within the request.
-// Elementwise, HBM-bound; one workgroup per token.  A thread owns one 16-byte
-// chunk column of the head dimension, evaluates its sin/cos once and walks the
-// heads, so the transcendental work is per (token, dim pair), not per head.
+// Elementwise, HBM-bound; one workgroup per token.  The token's sines and cosines are
+// evaluated once per (token, dim pair) into LDS; a thread owns one 16-byte chunk column
+// of the head dimension and walks the heads.
 #include "rope_math.h"
 
 namespace dskv {
@@ -18,6 +18,17 @@ struct AppendTarget {
     int num_pages;               // pages in the layer: an id outside [0, num_pages) is never written
 };
 
+// A chunk's tokens are a few rounds of workgroups on the chip, so the kernel lasts as long as a
+// workgroup's chain of dependent loads plus the copy itself.  The chain is kept short as in the
+// append kernel: the token's q, k (and v) chunks are requested first (their addresses need no
+// metadata: up to kRopeHeadsInFlight heads per thread are held in registers); the request that
+// owns the token comes from ONE vector load of qo_indptr and a ballot (lane i holds entry i;
+// batches of 64 requests or more take a binary search), with the request's offset, block-table
+// range and last-page length fetched by the same lanes at the same time; the page id is the
+// last link.
+constexpr int kRopeHeadsInFlight = 6;
+constexpr int kRopeMaxPairs = 1024;   // head_dim / 2 at most (a head row is at most 256 chunks of 16 bytes)
+
 template <int DT>
 __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, char *__restrict__ k_out,
                                                    const char *__restrict__ q,
@@ -30,55 +41,115 @@ __global__ __launch_bounds__(256) void rope_kernel(char *__restrict__ q_out, cha
     typedef Chunk<DT> C;
     constexpr int E = C::kElems;
     const int t = blockIdx.x;
-    int lo = 0, hi = batch;   // largest b with qo_indptr[b] <= t
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (qo_indptr[mid] <= t) lo = mid; else hi = mid;
+    const int lane = threadIdx.x & 63;
+    const int cols = head_dim / E;           // 16-byte chunks per head row
+    const int col = threadIdx.x % cols;
+    const int head_lane = threadIdx.x / cols;
+    const int head_lanes = 256 / cols;
+    const bool works = head_lane < head_lanes;   // the last threads of the workgroup may have no column
+    const long row_bytes = (long)head_dim * (16 / E);
+    const long kv_row_bytes = (long)n_kv_heads * row_bytes;
+    const int total_heads = n_qo_heads + n_kv_heads;
+    auto src_of = [&](int h) {
+        return h < n_qo_heads ? q + ((long)t * n_qo_heads + h) * row_bytes + col * 16
+                              : k + ((long)t * n_kv_heads + (h - n_qo_heads)) * row_bytes + col * 16;
+    };
+
+    // link 0: the rows themselves
+    u32x4 raw[kRopeHeadsInFlight], v_raw = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < kRopeHeadsInFlight; i++) {
+        const int h = head_lane + i * head_lanes;
+        if (works && h < total_heads) raw[i] = *reinterpret_cast<const u32x4 *>(src_of(h));
     }
-    if (t >= qo_indptr[lo + 1]) return;   // token not covered by the metadata
-    const float pos = (float)(offsets[lo] + (t - qo_indptr[lo]));
-    const long kv_row_bytes = (long)n_kv_heads * head_dim * (16 / E);
+    const char *v_src = tgt.pages ? tgt.v + (long)t * kv_row_bytes : nullptr;
+    if (v_src && threadIdx.x * 16L < kv_row_bytes) v_raw = *reinterpret_cast<const u32x4 *>(v_src + threadIdx.x * 16L);
+
+    // link 1: the request that owns token t = largest b with qo_indptr[b] <= t
+    int b, first, n_b, offset, page_begin = 0, n_pages = 0, last = 0;
+    if (batch < 64) {
+        const int i = min(lane, batch), j = min(lane, batch - 1);
+        const int q_i = qo_indptr[i];
+        const int o_i = offsets[j];
+        const int p_i = tgt.pages ? tgt.kv_indptr[i] : 0;
+        const int l_i = tgt.pages ? tgt.kv_last[j] : 0;
+        const unsigned long long le = __ballot(lane <= batch && q_i <= t);
+        b = min(__popcll(le) - 1, batch - 1);
+        if (b < 0) return;   // qo_indptr[0] > t: malformed
+        first = __shfl(q_i, b);
+        n_b = __shfl(q_i, b + 1) - first;
+        offset = __shfl(o_i, b);
+        page_begin = __shfl(p_i, b);
+        n_pages = __shfl(p_i, b + 1) - page_begin;
+        last = __shfl(l_i, b);
+    } else {
+        int lo = 0, hi = batch;
+        if (t < batch && qo_indptr[t] == t && qo_indptr[t + 1] == t + 1) {
+            lo = t;  // one token per request
+        } else {
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (qo_indptr[mid] <= t) lo = mid; else hi = mid;
+            }
+        }
+        b = lo;
+        first = qo_indptr[b];
+        n_b = qo_indptr[b + 1] - first;
+        offset = offsets[b];
+        if (tgt.pages) {
+            page_begin = tgt.kv_indptr[b];
+            n_pages = tgt.kv_indptr[b + 1] - page_begin;
+            last = tgt.kv_last[b];
+        }
+    }
+    if (t - first >= n_b) return;   // token not covered by the metadata
+    const float pos = (float)(offset + (t - first));
     char *k_dst = k_out + (long)t * kv_row_bytes;   // rotated K row set of this token
     char *v_dst = nullptr;
     if (tgt.pages) {
-        const int page_begin = tgt.kv_indptr[lo];
-        const int n_pages = tgt.kv_indptr[lo + 1] - page_begin;
-        const long kv_len = (long)(n_pages - 1) * tgt.page_size + tgt.kv_last[lo];
-        const long p = kv_len - (qo_indptr[lo + 1] - qo_indptr[lo]) + (t - qo_indptr[lo]);
+        const long kv_len = (long)(n_pages - 1) * tgt.page_size + last;
+        const long p = kv_len - n_b + (t - first);
         if (n_pages <= 0 || p < 0 || p >= kv_len) return;   // malformed metadata: touch nothing
+        // link 2: the page
         const long page = tgt.kv_indices[page_begin + (int)(p / tgt.page_size)];
         if (page < 0 || page >= tgt.num_pages) return;      // an id outside the pool: touch nothing
         const long half = (long)tgt.page_size * kv_row_bytes;
         k_dst = tgt.pages + page * 2 * half + (p % tgt.page_size) * kv_row_bytes;
         v_dst = k_dst + half;
     }
-
-    const int cols = head_dim / E;           // 16-byte chunks per head row
-    const int col = threadIdx.x % cols;
-    const int head_lane = threadIdx.x / cols;
-    const int head_lanes = 256 / cols;
-    if (head_lane >= head_lanes) return;
-
-    float cs[E / 2], sn[E / 2];
+    // cos and sin of the token's head_dim / 2 angles, each evaluated once per workgroup (a thread
+    // needs E / 2 of them, the same ones as every other thread of its column: evaluated per
+    // thread, the sincosf calls took as long as the kernel's memory traffic)
+    __shared__ float cos_of[kRopeMaxPairs], sin_of[kRopeMaxPairs];
+    for (int pair = threadIdx.x; pair < head_dim / 2; pair += 256)
+        rope_angle(pos, pair, head_dim, theta, freqs, cos_of[pair], sin_of[pair]);
+    __syncthreads();   // every exit above is taken by the whole workgroup or by none of it
+    if (works) {
+        float cs[E / 2], sn[E / 2];
 #pragma unroll
-    for (int j = 0; j < E / 2; j++) rope_angle(pos, col * (E / 2) + j, head_dim, theta, freqs, cs[j], sn[j]);
-    const long row_bytes = (long)head_dim * (16 / E);
-    const int total_heads = n_qo_heads + n_kv_heads;
-    for (int h = head_lane; h < total_heads; h += head_lanes) {
-        const bool is_q = h < n_qo_heads;
-        const long off = is_q ? ((long)t * n_qo_heads + h) * row_bytes
-                              : ((long)t * n_kv_heads + (h - n_qo_heads)) * row_bytes;
-        const char *src = (is_q ? q : k) + off + col * 16;
-        char *dst = is_q ? q_out + off + col * 16
-                         : k_dst + (long)(h - n_qo_heads) * row_bytes + col * 16;
-        float f[E];
-        C::unpack(*reinterpret_cast<const u32x4 *>(src), f);
-        rope_rotate<E / 2>(f, cs, sn);
-        *reinterpret_cast<u32x4 *>(dst) = C::pack(f);
+        for (int j = 0; j < E / 2; j++) {
+            cs[j] = cos_of[col * (E / 2) + j];
+            sn[j] = sin_of[col * (E / 2) + j];
+        }
+        auto rotate_into = [&](int h, const u32x4 &chunk) {
+            char *dst = h < n_qo_heads ? q_out + ((long)t * n_qo_heads + h) * row_bytes + col * 16
+                                       : k_dst + (long)(h - n_qo_heads) * row_bytes + col * 16;
+            float f[E];
+            C::unpack(chunk, f);
+            rope_rotate<E / 2>(f, cs, sn);
+            *reinterpret_cast<u32x4 *>(dst) = C::pack(f);
+        };
+#pragma unroll
+        for (int i = 0; i < kRopeHeadsInFlight; i++) {
+            const int h = head_lane + i * head_lanes;
+            if (h < total_heads) rotate_into(h, raw[i]);
+        }
+        for (int h = head_lane + kRopeHeadsInFlight * head_lanes; h < total_heads; h += head_lanes)
+            rotate_into(h, *reinterpret_cast<const u32x4 *>(src_of(h)));
     }
     if (v_dst) {   // fused append: V rows are copied as they are
-        const char *v_src = tgt.v + (long)t * kv_row_bytes;
-        for (long off = threadIdx.x * 16L; off < kv_row_bytes; off += 256 * 16)
+        if (threadIdx.x * 16L < kv_row_bytes) *reinterpret_cast<u32x4 *>(v_dst + threadIdx.x * 16L) = v_raw;
+        for (long off = threadIdx.x * 16L + 256 * 16; off < kv_row_bytes; off += 256 * 16)
             *reinterpret_cast<u32x4 *>(v_dst + off) = *reinterpret_cast<const u32x4 *>(v_src + off);
     }
 }
