@@ -467,6 +467,30 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
                        "rope_append_us_per_layer": round(rope_append_us, 1),
                        "rope_append_bytes": rope_append_bytes,
                        "rope_append_frac_of_hbm_peak": round(rope_append_bytes / rope_append_us / 1e3 / HBM_PEAK_GBPS, 4)}}
+    def sustained_attention():
+        for _ in range(8):
+            for layer in range(L):
+                w.forward(q[layer], pool.pages[layer], causal=True)
+
+    sensors = _BoardSensors()
+    if extras:
+        # the board's sensors while the attention launches run back to back for 3 s
+        r = _run_sampled(sensors, sustained_attention, 3.0, settle=1.0)
+        per_s = r.pop("launches_per_s")
+        # The first launches after a pause run in a transient of the board's power control (by
+        # rocprofv3 the first two dozen dispatches read 684, 689, 773, 828, 837, 810, ... 700 us
+        # before the kernel settles at 645-650 us): the figure above, a median over the first 20,
+        # is that transient; this one is the steady state, by the wall clock over two seconds.
+        if per_s:
+            sustained_us = 1e6 / (32 * per_s)
+            result.update({"attention_us_per_layer_sustained": round(sustained_us, 1),
+                           "attention_TFLOPs_sustained": round(flops / sustained_us / 1e6, 1),
+                           "frac_of_mfma_bf16_peak_sustained":
+                               round(flops / sustained_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4)})
+        result["power"] = {"what": "socket power and shader clock, sampled from the board's sensors while the "
+                                   "attention launches run back to back for 3 s (from second 1 on)",
+                           "power_cap_W": sensors.cap_watts(),
+                           "sustained_TFLOPs": round(32 * flops * per_s / 1e12, 1) if per_s else None, **r}
     if not extras:
         w.end_forward()
         return result
@@ -477,6 +501,9 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
     q.zero_()
     pool.pages.zero_()
     attn_zero_us = median_us(lambda layer: w.forward(q[layer], pool.pages[layer], causal=True))
+    r = _run_sampled(sensors, sustained_attention, 3.0, settle=1.0)
+    per_s = r.pop("launches_per_s")
+    result["power"]["zero_data"] = {"sustained_TFLOPs": round(32 * flops * per_s / 1e12, 1) if per_s else None, **r}
     w.end_forward()
     one_chunk = one_chunk_measure(gen)
     ceiling = mfma_ceiling_section(seed)
@@ -581,6 +608,47 @@ class _BoardSensors:
         return self._read(self.power, 1e6), clock if clock is not None else self._starred_mhz()
 
 
+def _run_sampled(sensors, launch, seconds: float, settle: float = 1.5):
+    """Calls launch() (which enqueues some 10-50 ms of work) and synchronizes, over and over for
+    `seconds`, while a thread samples the board's sensors every 50 ms; returns the launches per
+    second and the sensor averages from `settle` seconds on (clock and power have settled then)."""
+    import threading
+
+    import torch
+
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        t0 = time.perf_counter()
+        while not stop.is_set():
+            w_, f_ = sensors.sample()
+            samples.append((time.perf_counter() - t0, w_, f_))
+            time.sleep(0.05)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t0 = time.perf_counter()
+    n_settled, t_settled = 0, None
+    while time.perf_counter() - t0 < seconds:
+        launch()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 >= settle:
+            if t_settled is None:
+                t_settled = time.perf_counter()
+            else:
+                n_settled += 1
+    t_end = time.perf_counter()
+    stop.set()
+    th.join()
+    watts = [w_ for t_, w_, _ in samples if t_ >= settle and w_ is not None]
+    clocks = [f_ for t_, _, f_ in samples if t_ >= settle and f_ is not None]
+    return {"launches_per_s": n_settled / (t_end - t_settled) if t_settled and n_settled else None,
+            "socket_power_W_avg": round(sum(watts) / len(watts), 1) if watts else None,
+            "socket_power_W_max": round(max(watts), 1) if watts else None,
+            "shader_clock_MHz_avg": round(sum(clocks) / len(clocks), 1) if clocks else None,
+            "samples": len(watts)}
+
+
 def power_section(seed: int, seconds: float = 6.0):
     """Socket power and shader clock while a kernel runs back to back for `seconds` (sampled
     from the second 1.5 on, when clock and power have settled): the prefill attention of
@@ -588,7 +656,6 @@ def power_section(seed: int, seconds: float = 6.0):
     attention of configuration 2.  Says whether a kernel's rate is what the board's power cap
     leaves of the nominal clock."""
     import ctypes
-    import threading
 
     import numpy as np
     import torch
@@ -613,40 +680,11 @@ def power_section(seed: int, seconds: float = 6.0):
 
     def sustained(name, launch, work_per_launch, unit, what):
         """launch() enqueues some 10-50 ms of the kernel; work_per_launch in flop or bytes."""
-        samples, stop = [], threading.Event()
-
-        def sampler():
-            t0 = time.perf_counter()
-            while not stop.is_set():
-                w_, f_ = sensors.sample()
-                samples.append((time.perf_counter() - t0, w_, f_))
-                time.sleep(0.05)
-
-        th = threading.Thread(target=sampler, daemon=True)
-        th.start()
-        t0 = time.perf_counter()
-        n_settled, t_settled = 0, None
-        while time.perf_counter() - t0 < seconds:
-            launch()
-            torch.cuda.synchronize()
-            if time.perf_counter() - t0 >= 1.5:
-                if t_settled is None:
-                    t_settled = time.perf_counter()
-                else:
-                    n_settled += 1
-        t_end = time.perf_counter()
-        stop.set()
-        th.join()
-        watts = [w_ for t_, w_, _ in samples if t_ >= 1.5 and w_ is not None]
-        clocks = [f_ for t_, _, f_ in samples if t_ >= 1.5 and f_ is not None]
-        rate = work_per_launch * n_settled / (t_end - t_settled) if t_settled and n_settled else None
+        r = _run_sampled(sensors, launch, seconds)
+        rate = work_per_launch * r.pop("launches_per_s") if r["launches_per_s"] else None
         out["workloads"][name] = {
             "what": what,
-            "rate": round(rate / (1e12 if unit == "TFLOP/s" else 1e9), 1) if rate else None, "unit": unit,
-            "socket_power_W_avg": round(sum(watts) / len(watts), 1) if watts else None,
-            "socket_power_W_max": round(max(watts), 1) if watts else None,
-            "shader_clock_MHz_avg": round(sum(clocks) / len(clocks), 1) if clocks else None,
-            "samples": len(watts)}
+            "rate": round(rate / (1e12 if unit == "TFLOP/s" else 1e9), 1) if rate else None, "unit": unit, **r}
         time.sleep(1.0)           # let the board settle before the next workload
 
     # prefill attention, configuration 4 (as prefill_section builds it)
