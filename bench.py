@@ -510,6 +510,9 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
     measured_peak = ceiling["levels"]["mfma_only"]["normal"]
     result.update({"mfma_ceiling": ceiling,
                    "frac_of_measured_mfma_ceiling": round(result["attention_TFLOPs"] / measured_peak, 4),
+                   "frac_of_measured_mfma_ceiling_sustained":
+                       round(result["attention_TFLOPs_sustained"] / measured_peak, 4)
+                       if "attention_TFLOPs_sustained" in result else None,
                    "attention_us_per_layer_zero_data": round(attn_zero_us, 1),
                    "attention_TFLOPs_zero_data": round(flops / attn_zero_us / 1e6, 1),
                    "one_512_token_chunk_over_4096": one_chunk})
