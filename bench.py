@@ -433,11 +433,27 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
         ts = sorted(s.elapsed_time(e) for s, e in evs)
         return ts[len(ts) // 2] * 1e3
 
+    def back_to_back_us(fn, reps=8):
+        """All layers inside ONE bracket, `reps` times: the bracket's own 5-6 us (event and dispatch
+        latency), which a bracket around a single 12 us launch mostly measures, is spread over L."""
+        evs = []
+        for _ in range(reps):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for layer in range(L):
+                fn(layer)
+            e.record()
+            evs.append((s, e))
+        torch.cuda.synchronize()
+        ts = sorted(s.elapsed_time(e) for s, e in evs)
+        return ts[len(ts) // 2] * 1e3 / L
+
     def append(layer):
         append_paged_kv_cache(k[layer], v[layer], c.indptr, pool.pages[layer], c.kv_page_indices,
                               c.kv_page_indptr, c.kv_last_page_lens)
 
     append_us = median_us(append)
+    append_b2b_us = back_to_back_us(append)
     # the chunk's rotation: apply_rope alone, and rotation + append in one pass (what a layer
     # runs in front of the attention: q rotated out of place, rotated k and v into their slots)
     from deserve_amd.paged_ops import apply_rope, rope_append_paged_kv_cache
@@ -445,6 +461,11 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
     rope_us = median_us(lambda layer: apply_rope(q[layer], k[layer], c.indptr, offsets, interleave=True,
                                                  rope_theta=5e5))
     rope_append_us = median_us(lambda layer: rope_append_paged_kv_cache(
+        q[layer], k[layer], v[layer], c.indptr, offsets, pool.pages[layer], c.kv_page_indices,
+        c.kv_page_indptr, c.kv_last_page_lens, rope_theta=5e5))
+    rope_b2b_us = back_to_back_us(lambda layer: apply_rope(q[layer], k[layer], c.indptr, offsets, interleave=True,
+                                                           rope_theta=5e5))
+    rope_append_b2b_us = back_to_back_us(lambda layer: rope_append_paged_kv_cache(
         q[layer], k[layer], v[layer], c.indptr, offsets, pool.pages[layer], c.kv_page_indices,
         c.kv_page_indptr, c.kv_last_page_lens, rope_theta=5e5))
     append(0), append(1), append(2), append(3)          # the unrotated rows again, as the attention figures assume
@@ -456,6 +477,8 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
               "chunk_tokens": B * n, "kv_tokens": int((prior + n).sum()),
               "append_us_per_layer": round(append_us, 1),
               "append_GBps": round(2 * B * n * 2 * Hkv * D * 2 / append_us / 1e3, 1),
+              "append_us_per_layer_back_to_back": round(append_b2b_us, 1),
+              "append_GBps_back_to_back": round(2 * B * n * 2 * Hkv * D * 2 / append_b2b_us / 1e3, 1),
               "attention_us_per_layer": round(attn_us, 1),
               "attention_TFLOPs": round(flops / attn_us / 1e6, 1),
               "frac_of_mfma_bf16_peak": round(flops / attn_us / 1e6 / MFMA_PEAK_BF16_TFLOPS, 4),
@@ -466,7 +489,14 @@ def prefill_section(seed: int, extras: bool = True, config4: bool = True):
                        "apply_rope_frac_of_hbm_peak": round(rope_bytes / rope_us / 1e3 / HBM_PEAK_GBPS, 4),
                        "rope_append_us_per_layer": round(rope_append_us, 1),
                        "rope_append_bytes": rope_append_bytes,
-                       "rope_append_frac_of_hbm_peak": round(rope_append_bytes / rope_append_us / 1e3 / HBM_PEAK_GBPS, 4)}}
+                       "rope_append_frac_of_hbm_peak": round(rope_append_bytes / rope_append_us / 1e3 / HBM_PEAK_GBPS, 4),
+                       "back_to_back": {
+                           "what": "the 4 layers' launches inside one event bracket (the bracket's 5-6 us spread over 4)",
+                           "apply_rope_us_per_layer": round(rope_b2b_us, 1),
+                           "apply_rope_frac_of_hbm_peak": round(rope_bytes / rope_b2b_us / 1e3 / HBM_PEAK_GBPS, 4),
+                           "rope_append_us_per_layer": round(rope_append_b2b_us, 1),
+                           "rope_append_frac_of_hbm_peak":
+                               round(rope_append_bytes / rope_append_b2b_us / 1e3 / HBM_PEAK_GBPS, 4)}}}
     def sustained_attention():
         for _ in range(8):
             for layer in range(L):
