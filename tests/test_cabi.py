@@ -420,6 +420,118 @@ def test_mixed_plan_routes_one_row_requests_to_decode_items_and_tiles_the_rest(m
     assert info.tile_workspace_bytes >= (info.n_splits > 1) * 300 * info.n_splits * 32 * 130 * 4
 
 
+_RANDOM_PLAN_KINDS = {"shared": 0, "parts": 0, "cut_rows": 0}
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_mixed_plan_covers_every_row_exactly_once_on_random_batches(seed):
+    """Random ragged batches (one-row requests, empty requests, chunks, requests without kv
+    tokens; groups of 4 and 8; pages of 16 and 8 tokens) in every routing mode: each row of the
+    batch belongs to exactly one tile (whose parts partition its blocks) or to the decode work
+    list (whose items partition the row's kv tokens), never to both; partial slots never
+    overlap and lie inside the workspace the plan asks for; a shared plan's table of parts per
+    row agrees with both."""
+    lib = _lib.lib()
+    rng = np.random.default_rng(100 + seed)
+    n_req = int(rng.integers(1, 60))
+    # one row / no rows / a chunk / one row without kv; odd seeds: few chunks (tiles cut into parts)
+    kinds = rng.choice(4, size=n_req, p=[0.6, 0.05, 0.3, 0.05] if seed % 2 == 0 else [0.9, 0.03, 0.04, 0.03])
+    if seed % 2:
+        kinds[int(rng.integers(0, n_req))] = 2
+    qo_lens = [1 if k in (0, 3) else 0 if k == 1 else int(rng.integers(2, 700 if seed % 2 == 0 else 300)) for k in kinds]
+    kv_lens = [0 if k == 3 else q + int(rng.integers(0 if seed % 2 == 0 or q == 1 else 3000, 6000))
+               for k, q in zip(kinds, qo_lens)]
+    P = int(rng.choice([16, 8]))
+    hq = int(rng.choice([32, 64]))
+    slot_bytes = hq * 130 * 4
+    seen = _RANDOM_PLAN_KINDS
+    for mode in (_lib.ROUTE_OFF, _lib.ROUTE_AUTO, _lib.ROUTE_TWO_LAUNCHES, _lib.ROUTE_SHARED_LAUNCH):
+        target = int(rng.choice([0, 0, -1, 64]))
+        rc, info, plan, qo, indptr = _mixed_plan(lib, qo_lens, kv_lens, P=P, hq=hq, target=target, route=mode)
+        assert rc == 0, _lib.last_error()
+        seen["shared"] += info.layout == _lib.LAYOUT_SHARED
+        seen["parts"] += info.n_splits > 1
+        seen["cut_rows"] += info.n_decode_items > info.n_decode_rows
+        nnz = int(qo[-1])
+        assert info.n_decode_rows + info.n_tile_rows == nnz
+        covered = np.zeros(nnz, np.int32)
+        # tiles: rows [q0, q0 + rows_per_tile) of request b; the parts of a tile partition its blocks
+        tiles = plan[: 6 * info.n_tiles].reshape(-1, 6)
+        shared = info.layout == _lib.LAYOUT_SHARED
+        rows_per_tile = (4 if shared else 8) * 32 // (hq // 8)
+        tile_slots = info.tile_workspace_bytes // slot_bytes
+        used_slots = []
+        by_tile = {}
+        for b, q0, blk0, blk1, part_word, first_slot in tiles.tolist():
+            by_tile.setdefault((b, q0), []).append((blk0, blk1, part_word, first_slot))
+        for (b, q0), parts in by_tile.items():
+            n_rows = min(rows_per_tile, qo_lens[b] - q0)
+            assert 0 <= q0 < qo_lens[b] and q0 % rows_per_tile == 0 and n_rows >= 1
+            covered[qo[b] + q0: qo[b] + q0 + n_rows] += 1
+            parts.sort()
+            if len(parts) == 1:
+                assert parts[0][0] == 0 and parts[0][1] == 0x7FFFFFFF and parts[0][2] == -1
+            else:
+                assert len(parts) <= info.n_splits <= 8
+                assert parts[0][0] == 0 and parts[-1][1] == 0x7FFFFFFF
+                assert all(x[1] == y[0] and x[0] % 4 == 0 for x, y in zip(parts, parts[1:]))
+                assert sorted(w & 0xFF for _, _, w, _ in parts) == list(range(len(parts)))
+                assert {w >> 8 for _, _, w, _ in parts} == {len(parts)} and len({f for *_, f in parts}) == 1
+                used_slots.append((parts[0][3], parts[0][3] + n_rows * len(parts)))
+        assert all(hi <= tile_slots for _, hi in used_slots)
+        # the decode work list: items partition [0, kv_len) of every routed row
+        if info.n_decode_rows:
+            dp = plan[info.decode_plan_at:]
+            n_items, wgs, n_slots, batch = dp[:4].tolist()
+            assert (n_items, wgs, batch) == (info.n_decode_items, info.n_decode_workgroups, info.n_decode_rows)
+            req = dp[4 + wgs + 1: 4 + wgs + 1 + 2 * batch].reshape(-1, 2)
+            items = dp[4 + wgs + 1 + 2 * batch: 4 + wgs + 1 + 2 * batch + 8 * n_items].reshape(-1, 8)
+            row_map = plan[info.row_map_at: info.row_map_at + batch]
+            assert info.decode_workspace_bytes == n_slots * slot_bytes
+            routed = [b for b in range(n_req) if qo_lens[b] == 1 and kv_lens[b] > 0]
+            assert row_map.tolist() == [int(qo[b]) for b in routed]
+            for i, b in enumerate(routed):
+                covered[qo[b]] += 1
+                mine = items[items[:, 0] == qo[b]]
+                spans = sorted((t0, t1) for _, t0, t1, *_ in mine.tolist())
+                assert spans[0][0] == 0 and spans[-1][1] == kv_lens[b]
+                assert all(x[1] == y[0] for x, y in zip(spans, spans[1:]))
+                first, n = req[i].tolist()
+                assert (n == 0 and len(mine) == 1 and mine[0, 3] == -1) or \
+                       (n == len(mine) > 1 and sorted(mine[:, 3].tolist()) == list(range(first, first + n)))
+                if n:
+                    used_slots.append((tile_slots + first, tile_slots + first + n))
+            if shared:
+                both = plan[info.row_map_at + batch: info.plan_words].reshape(-1, 2)
+                assert both.shape[0] == nnz
+                for i, b in enumerate(routed):
+                    first, n = req[i].tolist()
+                    assert both[qo[b]].tolist() == ([tile_slots + first, n] if n else [0, 0])
+                for (b, q0), parts in by_tile.items():
+                    n_rows = min(rows_per_tile, qo_lens[b] - q0)
+                    for r in range(n_rows):
+                        want = [parts[0][3] + r * len(parts), len(parts)] if len(parts) > 1 else [0, 0]
+                        assert both[qo[b] + q0 + r].tolist() == want
+        else:
+            assert info.layout == _lib.LAYOUT_SEPARATE
+        assert (covered == 1).all(), (mode, np.flatnonzero(covered != 1)[:8])
+        used_slots.sort()
+        assert all(x[1] <= y[0] for x, y in zip(used_slots, used_slots[1:]))
+        if mode == _lib.ROUTE_OFF:
+            assert info.n_decode_rows == 0
+        if mode == _lib.ROUTE_SHARED_LAUNCH and info.n_decode_rows and info.n_tile_rows:
+            assert shared
+
+
+def test_random_mixed_plans_included_every_kind():
+    """The random batches above are worth their name only if shared launches, tiles in parts and
+    decode rows cut across workgroups all occur among them (run alone, this test draws them itself)."""
+    if not any(_RANDOM_PLAN_KINDS.values()):
+        for seed in range(12):
+            test_mixed_plan_covers_every_row_exactly_once_on_random_batches(seed)
+    assert all(v >= 3 for v in _RANDOM_PLAN_KINDS.values()), _RANDOM_PLAN_KINDS
+
+
 def test_mixed_plan_without_routing_is_the_prefill_plan():
     lib = _lib.lib()
     qo_lens, kv_lens = [1, 1, 200, 1], [700, 33, 900, 16]
