@@ -555,6 +555,57 @@ def test_mixed_batch_routes_one_row_requests_to_the_decode_kernel(case):
         w.end_forward()
 
 
+def test_mixed_batches_random_shapes():
+    """Seeded sweep over mixed batches (one-row requests with and without kv tokens, empty
+    requests, chunks), page sizes of 4 to 32 tokens, kv-head counts and groups, dtypes and the
+    four routing modes: every row of the NaN-filled output matches the oracle's prefill
+    attention.  The sweep must meet shared launches, tiles in parts and cut decode rows."""
+    from deserve_amd import _lib
+    from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
+
+    rng = np.random.default_rng(79)
+    w = BatchPrefillWithPagedKVCacheWrapper(torch.empty(128 << 20, dtype=torch.uint8, device="cuda"))
+    seen = {"shared": 0, "parts": 0, "cut_rows": 0, "two_launches": 0}
+    for done in range(24):
+        P = int(rng.choice([4, 8, 16, 32]))
+        Hkv = int(rng.choice([1, 2, 4, 8, 16]))
+        Hq = Hkv * int(rng.choice([1, 2, 4, 8]))
+        if Hq > 64:
+            Hq = 64
+        dtype = str(rng.choice(["bf16", "f16"]))
+        n_req = int(rng.integers(2, 24))
+        kinds = rng.choice(4, size=n_req, p=[0.7, 0.05, 0.2, 0.05])
+        kinds[0] = 2                                       # at least one chunk ...
+        kinds[1] = 0                                       # ... and one decode row
+        qo = [1 if k in (0, 3) else 0 if k == 1 else int(rng.integers(2, 200)) for k in kinds]
+        kv = [0 if k == 3 else n + int(rng.integers(0, 1500)) for k, n in zip(kinds, qo)]
+        if done % 3 == 0:
+            kv[0] += int(rng.integers(1500, 3000))         # a chunk behind a long context: tiles in parts
+        route = [_lib.ROUTE_SHARED_LAUNCH, _lib.ROUTE_TWO_LAUNCHES, True, False][done % 4]
+        target = int(rng.choice([0, 0, 48]))
+        causal = bool(rng.integers(0, 2))
+        _announce("mixed random", done, P, Hq, Hkv, dtype, route, target, causal, "qo", qo, "kv", kv)
+        sc = make_scenario(4000 + done, kv_lens=kv, qo_lens=qo, P=P, Hq=Hq, Hkv=Hkv, D=128, dtype=dtype)
+        w.begin_forward(_dev_i32(sc.qo_indptr), _dev_i32(sc.kv_page_indptr), _dev_i32(sc.kv_page_indices),
+                        _dev_i32(sc.kv_last_page_lens), Hq, Hkv, 128, P, target_workgroups=target,
+                        route_one_row_requests=route)
+        seen["shared"] += w._info.layout == _lib.LAYOUT_SHARED
+        seen["two_launches"] += w._info.layout != _lib.LAYOUT_SHARED and w._n_decode_rows > 0 and w._info.n_tile_rows > 0
+        seen["parts"] += w._n_splits > 1
+        seen["cut_rows"] += w._info.n_decode_items > w._n_decode_rows
+        q, pages = to_torch(sc.q, dtype), to_torch(sc.pages, dtype)
+        out = torch.full_like(q, float("nan"))
+        w.forward(q, pages, causal=causal, out=out)
+        w.end_forward()
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        want = c_oracle.prefill_attn(sc.q, sc.qo_indptr, sc.pages, sc.kv_page_indices, sc.kv_page_indptr,
+                                     sc.kv_last_page_lens, dtype, causal=causal)
+        assert np.isfinite(got).all(), (done, route)
+        assert max_rel_err_per_request(got, want) <= ATTN_TOL[dtype], (done, P, Hq, Hkv, dtype, route, qo, kv)
+    assert all(v >= 2 for v in seen.values()), seen
+
+
 def test_prefill_with_one_query_equals_decode():
     from deserve_amd.paged_ops import BatchPrefillWithPagedKVCacheWrapper
 
