@@ -403,19 +403,21 @@ def test_mixed_step_full_size_through_batch_prefill():
     over a prior of U[0, 4096] tokens, all through BatchPrefill (engine/microbatch/processor.py:
     116-145) at the Llama-3-8B stage shape (the chunk behind 4200 tokens, its tiles in parts)
     and at the 70B shape (behind 1500 tokens) - the planner runs both as one launch in which
-    decode workgroups and query tiles share the compute units - and a step of 8 running requests
-    and a 504-token chunk, which it runs as tiles only.  EVERY row of the ragged output of
+    decode workgroups and query tiles share the compute units, as it does the 8B step in f16 on
+    pages of 8 tokens - and a step of 8 running requests and a 504-token chunk, which it runs
+    as tiles only.  EVERY row of the ragged output of
     two layers against the C oracle, each row against its own scale; the appended rows read
     back bit for bit; the layer's checksum moves by exactly the appended rows."""
     from deserve_amd.execution.exec import BatchPrefill, get_wrappers
     from deserve_amd.synthetic import make_mixed_workload, mixed_step_shape
 
-    for tag, L, Hq in (("8B", 3, 32), ("70B", 2, 64), ("8B_few_rows", 2, 32)):
+    for tag, L, Hq in (("8B", 3, 32), ("70B", 2, 64), ("8B_few_rows", 2, 32), ("8B_page8_f16", 2, 32)):
         _announce("mixed step", tag)
-        P, Hkv, D = 16, 8, 128
+        P, Hkv, D = (8 if tag == "8B_page8_f16" else 16), 8, 128          # 8 tokens: the page the reference deploys with
+        dtype, dtype_name = (torch.float16, "f16") if tag == "8B_page8_f16" else (torch.bfloat16, "bf16")
         dctx, prior, lens = mixed_step_shape(11, decode_rows=8 if tag == "8B_few_rows" else 75)
         prior[0] = 4200 if tag == "8B" else 1500
-        wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, torch.bfloat16, seed=11)
+        wl = make_mixed_workload("mixed" + tag, dctx, prior, lens, L, Hq, Hkv, D, P, dtype, seed=11)
         nnz, n_dec = wl.nnz, len(dctx)
         assert nnz == 512
         before = [_checksum(wl.pool.pages[l]) for l in range(L)]
@@ -448,7 +450,7 @@ def test_mixed_step_full_size_through_batch_prefill():
         for l in (0, L - 1):
             pages = _bits(wl.pool.pages[l].index_select(0, torch.from_numpy(ids_all.astype(np.int64)).to(DEV)))
             want = c_oracle.prefill_attn(_bits(wl.q[l]), qo, pages, np.arange(len(ids_all), dtype=np.int32),
-                                         indptr, last, "bf16", causal=True)
+                                         indptr, last, dtype_name, causal=True)
             got = result[l].view(nnz, Hq, D).float().cpu().numpy()
             assert np.isfinite(got).all()
             err_dec = max_rel_err_per_request(got[:n_dec], want[:n_dec])
