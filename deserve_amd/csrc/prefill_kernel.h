@@ -30,6 +30,9 @@ constexpr int kStageBytes = (kBlock / 4) * kRegionBytes;
 // than this (log2 domain): probabilities stay below 2^8, the accumulators are
 // rescaled a handful of times per query instead of once per block.
 constexpr float kRescaleSlack = 8.f;
+#ifndef DSKV_PREFILL_KPREFETCH
+#define DSKV_PREFILL_KPREFETCH 1   // K operands of the next iteration read before its barrier (direct path)
+#endif
 #ifndef DSKV_PREFILL_KREADS_FIRST
 #define DSKV_PREFILL_KREADS_FIRST 0
 #endif
@@ -304,14 +307,18 @@ __device__ __forceinline__ void prefill_attn_body(
     // P(m) while S(m+1) is computed): the loop is unrolled with static phases, so which
     // buffer is which is known at compile time and no copy is needed.
     f32x16 xs[2][kColTiles];
-    u32x4 ka[8];   // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7
-    auto read_k_operands = [&](const char *kst) {
+    // K rows of a block as MFMA operands: token r, dims 16*ks + 8h .. +7.  With the prefetch
+    // the operands of K(m+1) are read at the end of iteration m-1 (the block has been published
+    // by barrier m-1 then), into the buffer that iteration m's scores use; without, all use [0].
+    constexpr bool kKPrefetch = DSKV_PREFILL_KPREFETCH && kRowsSharePage;
+    u32x4 ka[kKPrefetch ? 2 : 1][8];
+    auto read_k_operands = [&](const char *kst, int kb = 0) {
         // token r = row r & 3 of region r >> 2; chunk 2 ks + h
         const char *k_rows = kst + (r >> 2) * kRegionBytes + h * 64 + (r & 3) * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) ka[ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 128);
+        for (int ks = 0; ks < 8; ks++) ka[kb][ks] = *reinterpret_cast<const u32x4 *>(k_rows + ks * 128);
     };
-    auto scores = [&](int buf) {
+    auto scores = [&](int buf, int kb = 0) {
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++)
 #pragma unroll
@@ -320,7 +327,7 @@ __device__ __forceinline__ void prefill_attn_body(
         for (int ks = 0; ks < 8; ks++)
 #pragma unroll
             for (int ct = 0; ct < kColTiles; ct++)
-                xs[buf][ct] = E::mfma_32x32(ka[ks], qreg[ct][ks], xs[buf][ct]);
+                xs[buf][ct] = E::mfma_32x32(ka[kb][ks], qreg[ct][ks], xs[buf][ct]);
     };
     // Masks block blk's scores (needed from w_mask_from on).  The empty volatile statement
     // keeps this a branch: the compiler otherwise turns it into selects that every block
@@ -363,13 +370,17 @@ __device__ __forceinline__ void prefill_attn_body(
     // Block j lives in K stage j % 4 and V stage j % 4.  Per iteration one barrier; every
     // wave runs every iteration (idle ones only move rows), so the barriers match.  The loop
     // is unrolled by four so that all stage indices are static.
-    //   Direct path: iteration m requests K(m+3) and V(m+2) behind its barrier (K(m+3)
-    //   replaces K(m-1), last read in iteration m-2; V(m+2) replaces V(m-2), last read in
-    //   iteration m-1).  K(m+1), which iteration m reads, went out two iterations earlier; a
-    //   wave makes sure that its own part of it has landed (at most 3 younger loads per row
-    //   group outstanding: V(m), K(m+2), V(m+1)) before it joins the barrier
-    //   that publishes the block.  The page of block j is looked up in iteration j-5 and its
-    //   descriptors are built in iteration j-4, behind that iteration's MFMAs.
+    //   Direct path: iteration m requests K(m+4) and V(m+2) behind its barrier (K(m+4)
+    //   replaces K(m), whose operands were read at the end of iteration m-2; V(m+2) replaces
+    //   V(m-2), last read in iteration m-1).  The operands of K(m+1) are read at the END of
+    //   iteration m-1, into the registers iteration m's score MFMAs use, so that those MFMAs
+    //   start right behind the barrier instead of waiting for LDS (steady state +0.65 %); for
+    //   that K(m+2) must have been published by barrier m: it went out two iterations
+    //   earlier, and a wave makes sure that its own part of it has landed (at most 3 younger
+    //   loads per row group outstanding: V(m), K(m+3), V(m+1)) before it joins that barrier.
+    //   The page of block j is looked up in iteration j-6 and its descriptors are built in
+    //   iteration j-5, behind that iteration's MFMAs.  (DSKV_PREFILL_KPREFETCH=0: the operands
+    //   of K(m+1) are read at the start of iteration m, every request one block nearer.)
     //   Register path: the rows of block m+4 are requested in iteration m and written to
     //   LDS in iteration m+2 (one iteration is shorter than a trip to memory).
     RowDesc desc[4];              // descriptors of block j in desc[j % 4]
@@ -391,10 +402,14 @@ __device__ __forceinline__ void prefill_attn_body(
 #pragma unroll
             for (int blk = 0; blk < 4; blk++) prepare_rows(blk_begin + blk, pg[blk], desc[blk]);
 #pragma unroll
-            for (int blk = 0; blk < 3; blk++) load_direct(desc[blk].k, k_stage[blk]);
+            for (int blk = 0; blk < (kKPrefetch ? 4 : 3); blk++) load_direct(desc[blk].k, k_stage[blk]);
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) load_direct(desc[blk].v, v_stage[blk]);
             lookup_pages(blk_begin + 4, pg[0]);
+            if (kKPrefetch) {   // one block further ahead: block 4's descriptors now, block 5's page
+                prepare_rows(blk_begin + 4, pg[0], desc[0]);
+                lookup_pages(blk_begin + 5, pg[1]);
+            }
             DSKV_WAIT_VMEM(0);
         } else {
             u32x4 first_k[2][kRowGroups], first_v[2][kRowGroups];
@@ -411,10 +426,11 @@ __device__ __forceinline__ void prefill_attn_body(
     }
     __syncthreads();
     if (w_end > 0) {
-        read_k_operands(k_stage[0]);
-        scores(0);
+        read_k_operands(k_stage[0], kKPrefetch ? 1 : 0);
+        scores(0, kKPrefetch ? 1 : 0);
         if ((blk_begin + 1) * kBlock > w_mask_from) mask_scores(blk_begin, 0);
         block_max(0);
+        if (kKPrefetch) read_k_operands(k_stage[1], 0);   // K(blk_begin + 1) for the first iteration
     }
     // V operand: token 16 ks + 8 hi + 4 h + (c >> 2) = row c >> 2 of region 4 ks + 2 hi + h;
     // bytes 64 dt + 32 (g & 1) + 8 (c & 3) of its row = half (c & 1) of chunk 4 dt + 2 (g & 1) + ((c & 3) >> 1)
@@ -436,7 +452,11 @@ __device__ __forceinline__ void prefill_attn_body(
         } else {
             __syncthreads();
         }
-        if (kRowsSharePage) {
+        if (kRowsSharePage && kKPrefetch) {
+            lookup_pages(m + 6, pg[(phase + 2) & 3]);
+            load_direct(desc[phase].k, k_stage[phase]);                       // K(m+4) over K(m), read in iteration m-2
+            load_direct(desc[(phase + 2) & 3].v, v_stage[(phase + 2) & 3]);   // V(m+2)
+        } else if (kRowsSharePage) {
             lookup_pages(m + 5, pg[(phase + 1) & 3]);
             load_direct(desc[(phase + 3) & 3].k, k_stage[(phase + 3) & 3]);   // K(m+3)
             load_direct(desc[(phase + 2) & 3].v, v_stage[(phase + 2) & 3]);   // V(m+2)
@@ -446,7 +466,8 @@ __device__ __forceinline__ void prefill_attn_body(
             load_rows(m + 4, rows.k, rows.v);
         }
         if (!(w_end > 0 && (m - 1) * kBlock < w_end)) {
-            prepare_rows(m + 4, pg[phase], desc[phase]);
+            if (kKPrefetch) prepare_rows(m + 5, pg[(phase + 1) & 3], desc[(phase + 1) & 3]);
+            else prepare_rows(m + 4, pg[phase], desc[phase]);
             return;
         }
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
@@ -489,7 +510,7 @@ __device__ __forceinline__ void prefill_attn_body(
         // V operand: the transposing read hands each block of 16 lanes four tokens
         // of 16 consecutive dims, lane i of the block supplying the address of dims
         // 4*(i%4) .. +3 of the block's token i/4
-        read_k_operands(k_stage[(phase + 1) & 3]);                       // K(m+1)
+        if (!kKPrefetch) read_k_operands(k_stage[(phase + 1) & 3]);      // K(m+1)
 #if DSKV_PREFILL_KREADS_FIRST
         __builtin_amdgcn_sched_barrier(0);   // all eight K operands requested before anything else
 #endif
@@ -504,7 +525,7 @@ __device__ __forceinline__ void prefill_attn_body(
                 const u32x2 a_hi = read_transposed(vp + 2 * kRegionBytes);
                 va[dt][ks] = u32x4{a_lo.x, a_lo.y, a_hi.x, a_hi.y};
             }
-        scores(nxt);
+        scores(nxt, kKPrefetch ? (phase & 1) : 0);
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) {
             float p[16], p_sum = 0.f;
@@ -536,7 +557,12 @@ __device__ __forceinline__ void prefill_attn_body(
 #pragma unroll
                 for (int ct = 0; ct < kColTiles; ct++)
                     l_acc[ct] = E::mfma_32x32(ones, pb_prev[ct][ks], l_acc[ct]);
-        prepare_rows(m + 4, pg[phase], desc[phase]);   // for the loads of the next iterations
+        if (kKPrefetch) {
+            read_k_operands(k_stage[(phase + 2) & 3], (phase + 1) & 1);   // K(m+2), published by this iteration's barrier
+            prepare_rows(m + 5, pg[(phase + 1) & 3], desc[(phase + 1) & 3]);
+        } else {
+            prepare_rows(m + 4, pg[phase], desc[phase]);   // for the loads of the next iterations
+        }
         block_max(nxt);
 #pragma unroll
         for (int ct = 0; ct < kColTiles; ct++) asm volatile("" ::"v"(m_blk[ct]));
